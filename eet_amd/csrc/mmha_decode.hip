@@ -1,0 +1,352 @@
+// Masked multi-head decode attention over the fp16 KV cache (one new token per
+// sequence), with an optional ALiBi bias row.
+//
+// Replaces masked_attention_kernel_opt (csrc/core/attention_dispatch.cu:140-324,
+// dispatcher :888-928) and t5_masked_attention_kernel (:1155-1336, dispatcher
+// :1397-1424).  Semantics kept: logit = (q . k_t) * half(1/sqrt(dh)) [+ bias],
+// rows t < pad[b] carry no weight, softmax denominator + 1e-6, fp32 math.
+// Not kept: the reference rounds each logit to fp16 (:238) and caps step at
+// 4096 by a static shared array (:164).
+//
+// HBM-bound: K and V rows (dh halves, contiguous) are each read exactly once
+// with 128-bit loads.  The cache is [B_cap][H][T_cap][dh], so one (b, h) pair
+// streams one contiguous range.  The time axis is split over `nsplit`
+// workgroups per (b, h) so that a few hundred heads still fill 256 CUs
+// (the reference runs one block per head); every workgroup produces an
+// un-normalised partial (max, sum, acc[dh]) and a second small kernel merges
+// them.  With nsplit == 1 the first kernel writes the context itself.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "common.h"
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kMaxChunk = 2048;  // logits of one workgroup's time range, kept in LDS
+
+__device__ __forceinline__ float dot8(const u32x4 &a, const u32x4 &b)
+{
+    const half8 ha = __builtin_bit_cast(half8, a), hb = __builtin_bit_cast(half8, b);
+    float s = 0.f;
+    s = __builtin_amdgcn_fdot2(__builtin_shufflevector(ha, ha, 0, 1), __builtin_shufflevector(hb, hb, 0, 1), s, false);
+    s = __builtin_amdgcn_fdot2(__builtin_shufflevector(ha, ha, 2, 3), __builtin_shufflevector(hb, hb, 2, 3), s, false);
+    s = __builtin_amdgcn_fdot2(__builtin_shufflevector(ha, ha, 4, 5), __builtin_shufflevector(hb, hb, 4, 5), s, false);
+    s = __builtin_amdgcn_fdot2(__builtin_shufflevector(ha, ha, 6, 7), __builtin_shufflevector(hb, hb, 6, 7), s, false);
+    return s;
+}
+
+// Decode streams every cache row once (non-temporal); the prompt pass re-reads
+// rows for every query, so it keeps them cacheable.
+template <bool STREAM>
+__device__ __forceinline__ u32x4 load_row16(const u32x4 *p)
+{
+    return STREAM ? __builtin_nontemporal_load(p) : *p;
+}
+
+template <int WIDTH>
+__device__ __forceinline__ float group_sum(float v)
+{
+#pragma unroll
+    for (int off = WIDTH / 2; off > 0; off >>= 1)
+        v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ float block_reduce(float v, bool is_max, float *scratch)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        float o = __shfl_xor(v, off, 64);
+        v = is_max ? fmaxf(v, o) : v + o;
+    }
+    if (lane == 0)
+        scratch[wave] = v;
+    __syncthreads();
+    float r = scratch[0];
+#pragma unroll
+    for (int w = 1; w < kThreads / 64; ++w)
+        r = is_max ? fmaxf(r, scratch[w]) : r + scratch[w];
+    __syncthreads();
+    return r;
+}
+
+// DH: head size.  LPR = DH/8 lanes cover one row with one 16-byte load each.
+// PREFILL = false: one query per (b, h), rows [0, step).
+// PREFILL = true : blockIdx.x also runs over the S = step prompt positions;
+//   query i of q[B][H][S][dh] attends rows [0, i] and writes ctx[b][i][h*dh..]
+//   (the causal prompt pass, one workgroup per query row; nsplit is 1).
+template <int DH, bool PREFILL>
+__global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
+    const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_new, const _Float16 *__restrict__ v_new,
+    long qkv_stride, _Float16 *__restrict__ k_cache, _Float16 *__restrict__ v_cache, _Float16 *__restrict__ ctx,
+    const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, float *__restrict__ partial, int H,
+    int step_or_S, int T_cap, int nsplit, float scale)
+{
+    constexpr int LPR = DH / 8;            // lanes per row
+    constexpr int RPB = kThreads / LPR;    // rows in flight per pass of the block
+    __shared__ float logits[kMaxChunk];
+    __shared__ float red[kThreads / 64];
+    __shared__ float accs[RPB][DH + 1];
+
+    const int split = blockIdx.y;
+    const int bh = PREFILL ? blockIdx.x / step_or_S : blockIdx.x;
+    const int qi = PREFILL ? blockIdx.x % step_or_S : 0;
+    const int step = PREFILL ? qi + 1 : step_or_S;
+    const int alibi_ld = step_or_S;
+    const int b = bh / H, h = bh % H;
+    const int tid = threadIdx.x;
+    const int sub = tid % LPR;   // which 8-element slice of the row
+    const int rs = tid / LPR;    // which row stream
+
+    const size_t qoff = PREFILL ? (size_t)blockIdx.x * DH
+                                : (qkv_stride ? (size_t)b * qkv_stride + (size_t)h * DH : (size_t)bh * DH);
+    const size_t coff = PREFILL ? ((size_t)(b * step_or_S + qi) * H + h) * DH : (size_t)bh * DH;
+    _Float16 *kc = k_cache + ((size_t)b * H + h) * (size_t)T_cap * DH;
+    _Float16 *vc = v_cache + ((size_t)b * H + h) * (size_t)T_cap * DH;
+
+    int t_first = pad ? (int)min((int64_t)step, max((int64_t)0, pad[b])) : 0;
+    if (PREFILL && pad && (int64_t)qi < pad[b])
+        t_first = step;  // a padded query row attends nothing and yields zeros
+    const int span = step - t_first;
+    const int per = (span + nsplit - 1) / nsplit;
+    const int t0 = t_first + split * per;
+    const int t1 = min(step, t0 + per);
+    const int n = max(0, t1 - t0);
+
+    // Append the new token's k, v (row step-1).  Only the workgroup that owns
+    // that row writes it, then reads it back like any other row.
+    if (k_new != nullptr && step - 1 >= t0 && step - 1 < t1) {
+        if (tid < LPR) {
+            *reinterpret_cast<uint4 *>(kc + (size_t)(step - 1) * DH + tid * 8) =
+                *reinterpret_cast<const uint4 *>(k_new + qoff + tid * 8);
+        } else if (tid < 2 * LPR) {
+            const int s2 = tid - LPR;
+            *reinterpret_cast<uint4 *>(vc + (size_t)(step - 1) * DH + s2 * 8) =
+                *reinterpret_cast<const uint4 *>(v_new + qoff + s2 * 8);
+        }
+        __threadfence();
+    }
+    __syncthreads();
+
+    const u32x4 qv = *reinterpret_cast<const u32x4 *>(q + qoff + sub * 8);
+
+    // Phase 1: logits of rows [t0, t1).
+    float lmax = -INFINITY;
+    for (int r0 = 0; r0 < n; r0 += RPB * 4) {
+        u32x4 kv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int r = r0 + u * RPB + rs;
+            if (r < n)
+                kv[u] = load_row16<!PREFILL>(reinterpret_cast<const u32x4 *>(kc + (size_t)(t0 + r) * DH) + sub);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int r = r0 + u * RPB + rs;
+            float d = (r < n) ? dot8(qv, kv[u]) : 0.f;
+            d = group_sum<LPR>(d) * scale;
+            if (r < n) {
+                if (alibi)
+                    d += (float)alibi[(size_t)h * alibi_ld + t0 + r];
+                if (sub == 0)
+                    logits[r] = d;
+                lmax = fmaxf(lmax, d);
+            }
+        }
+    }
+    lmax = block_reduce(lmax, true, red);  // also orders the logits[] writes
+
+    // Phase 2: un-normalised weights and their sum.
+    float lsum = 0.f;
+    for (int r = tid; r < n; r += kThreads) {
+        float p = __expf(logits[r] - lmax);
+        logits[r] = p;
+        lsum += p;
+    }
+    lsum = block_reduce(lsum, false, red);
+
+    // Phase 3: acc = sum_t p_t * v_t.
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int r0 = 0; r0 < n; r0 += RPB * 4) {
+        u32x4 vv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int r = r0 + u * RPB + rs;
+            if (r < n)
+                vv[u] = load_row16<!PREFILL>(reinterpret_cast<const u32x4 *>(vc + (size_t)(t0 + r) * DH) + sub);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int r = r0 + u * RPB + rs;
+            if (r < n) {
+                const float p = logits[r];
+                const half8 hv = __builtin_bit_cast(half8, vv[u]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    acc[e] += p * (float)hv[e];
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+        accs[rs][sub * 8 + e] = acc[e];
+    __syncthreads();
+    if (tid < DH) {
+        float s = 0.f;
+#pragma unroll 4
+        for (int r = 0; r < RPB; ++r)
+            s += accs[r][tid];
+        if (nsplit == 1) {
+            // n == 0 (everything padded away) gives 0 / 1e-6 = 0.
+            ctx[coff + tid] = (_Float16)(s / (lsum + 1e-6f));
+        } else {
+            float *p = partial + ((size_t)bh * nsplit + split) * (DH + 2);
+            p[2 + tid] = s;
+            if (tid == 0) {
+                p[0] = lmax;
+                p[1] = lsum;
+            }
+        }
+    }
+}
+
+template <int DH>
+__global__ __launch_bounds__(DH) void mmha_decode_merge_kernel(const float *__restrict__ partial,
+                                                               _Float16 *__restrict__ ctx, int nsplit)
+{
+    const int bh = blockIdx.x, tid = threadIdx.x;
+    const float *p = partial + (size_t)bh * nsplit * (DH + 2);
+    float m = -INFINITY;
+    for (int s = 0; s < nsplit; ++s)
+        m = fmaxf(m, p[s * (DH + 2)]);
+    float sum = 0.f, acc = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+        const float ms = p[s * (DH + 2)];
+        const float w = (ms == -INFINITY) ? 0.f : __expf(ms - m);
+        sum += w * p[s * (DH + 2) + 1];
+        acc += w * p[s * (DH + 2) + 2 + tid];
+    }
+    ctx[(size_t)bh * DH + tid] = (_Float16)(acc / (sum + 1e-6f));
+}
+
+int pick_nsplit(int BH, int step)
+{
+    // enough workgroups for ~4 per CU, at least 64 rows each, and no more rows
+    // per workgroup than the LDS logits array holds
+    int want = (1024 + BH - 1) / BH;
+    int by_rows = (step + 63) / 64;
+    int ns = want < by_rows ? want : by_rows;
+    int need = (step + kMaxChunk - 1) / kMaxChunk;
+    if (ns < need)
+        ns = need;
+    return ns < 1 ? 1 : ns;
+}
+
+template <int DH>
+int launch(const void *q, const void *k, const void *v, long qkv_stride, void *kc, void *vc, void *ctx,
+           const void *alibi, const int64_t *pad, int B, int H, int step, int T_cap, void *ws, int nsplit,
+           hipStream_t st)
+{
+    const float scale = (float)(_Float16)(1.0f / sqrtf((float)DH));
+    dim3 grid(B * H, nsplit);
+    hipLaunchKernelGGL((mmha_decode_split_kernel<DH, false>), grid, dim3(kThreads), 0, st,
+                       static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(k),
+                       static_cast<const _Float16 *>(v), qkv_stride, static_cast<_Float16 *>(kc),
+                       static_cast<_Float16 *>(vc), static_cast<_Float16 *>(ctx),
+                       static_cast<const _Float16 *>(alibi), pad, static_cast<float *>(ws), H, step, T_cap, nsplit,
+                       scale);
+    EET_HIP_CHECK(hipGetLastError());
+    if (nsplit > 1) {
+        hipLaunchKernelGGL((mmha_decode_merge_kernel<DH>), dim3(B * H), dim3(DH), 0, st,
+                           static_cast<const float *>(ws), static_cast<_Float16 *>(ctx), nsplit);
+        EET_HIP_CHECK(hipGetLastError());
+    }
+    return EET_OK;
+}
+
+template <int DH>
+int launch_prefill(const void *q, const void *kc, const void *vc, void *ctx, const void *alibi, const int64_t *pad,
+                   int B, int H, int S, int T_cap, hipStream_t st)
+{
+    const float scale = (float)(_Float16)(1.0f / sqrtf((float)DH));
+    hipLaunchKernelGGL((mmha_decode_split_kernel<DH, true>), dim3((unsigned)(B * H * S), 1), dim3(kThreads), 0, st,
+                       static_cast<const _Float16 *>(q), nullptr, nullptr, 0L,
+                       static_cast<_Float16 *>(const_cast<void *>(kc)),
+                       static_cast<_Float16 *>(const_cast<void *>(vc)), static_cast<_Float16 *>(ctx),
+                       static_cast<const _Float16 *>(alibi), pad, nullptr, H, S, T_cap, 1, scale);
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
+}  // namespace
+
+// Interim prompt pass: one workgroup per query row re-using the decode kernel
+// (K and V rows are re-read per query from L2).  Correct, not fast.
+extern "C" int eet_prefill_attention(const void *q, const void *k_cache, const void *v_cache, void *ctx,
+                                     const void *alibi, const int64_t *pad, int B, int H, int S, int dh, int T_cap,
+                                     void *stream)
+{
+    EET_REQUIRE(q && k_cache && v_cache && ctx, EET_ERR_INVALID_ARGUMENT, "eet_prefill_attention: null pointer");
+    EET_REQUIRE(B > 0 && H > 0 && S > 0 && S <= T_cap, EET_ERR_INVALID_ARGUMENT,
+                "eet_prefill_attention: bad sizes B=%d H=%d S=%d T_cap=%d", B, H, S, T_cap);
+    EET_REQUIRE(dh == 32 || dh == 64 || dh == 128, EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_prefill_attention: head size %d not supported (32, 64, 128)", dh);
+    EET_REQUIRE(S <= kMaxChunk, EET_ERR_UNSUPPORTED_SHAPE, "eet_prefill_attention: prompt length %d exceeds %d", S,
+                kMaxChunk);
+    EET_REQUIRE((long long)B * H * S < (1LL << 31), EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_prefill_attention: B*H*S too large");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dh) {
+        case 32: return launch_prefill<32>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
+        case 64: return launch_prefill<64>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
+        default: return launch_prefill<128>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
+    }
+}
+
+extern "C" size_t eet_mmha_decode_workspace(int B, int H, int dh, int step)
+{
+    if (B <= 0 || H <= 0 || dh <= 0 || step <= 0)
+        return 0;
+    const int ns = pick_nsplit(B * H, step);
+    return ns > 1 ? (size_t)B * H * ns * (dh + 2) * sizeof(float) : 0;
+}
+
+extern "C" int eet_mmha_decode(const void *q, const void *k, const void *v, long qkv_stride, void *k_cache,
+                               void *v_cache, void *ctx, const void *alibi, const int64_t *pad, int B, int H,
+                               int dh, int step, int T_cap, void *workspace, size_t workspace_bytes, void *stream)
+{
+    EET_REQUIRE(q && k_cache && v_cache && ctx, EET_ERR_INVALID_ARGUMENT, "eet_mmha_decode: null pointer");
+    EET_REQUIRE((k == nullptr) == (v == nullptr), EET_ERR_INVALID_ARGUMENT,
+                "eet_mmha_decode: k and v must both be given or both be NULL");
+    EET_REQUIRE(B > 0 && H > 0 && step > 0 && T_cap > 0, EET_ERR_INVALID_ARGUMENT,
+                "eet_mmha_decode: bad sizes B=%d H=%d step=%d T_cap=%d", B, H, step, T_cap);
+    EET_REQUIRE(step <= T_cap, EET_ERR_INVALID_ARGUMENT, "eet_mmha_decode: step %d exceeds the cache capacity %d",
+                step, T_cap);
+    EET_REQUIRE(dh == 32 || dh == 64 || dh == 128, EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_mmha_decode: head size %d not supported (32, 64, 128)", dh);
+    EET_REQUIRE(qkv_stride >= 0 && qkv_stride % 8 == 0, EET_ERR_INVALID_ARGUMENT,
+                "eet_mmha_decode: qkv_stride must be a non-negative multiple of 8");
+    const int ns = pick_nsplit(B * H, step);
+    const size_t need = eet_mmha_decode_workspace(B, H, dh, step);
+    EET_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), EET_ERR_WORKSPACE,
+                "eet_mmha_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dh) {
+        case 32:
+            return launch<32>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, workspace,
+                              ns, st);
+        case 64:
+            return launch<64>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, workspace,
+                              ns, st);
+        default:
+            return launch<128>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap,
+                               workspace, ns, st);
+    }
+}

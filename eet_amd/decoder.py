@@ -1,0 +1,184 @@
+"""Caller of the operator API: a LLaMA- / Baichuan-shaped int8 decoder assembled
+from the ops exactly as the reference's Python model code assembles it, plus
+the greedy loop that drives it.
+
+Counterpart of python/eet/transformers/modeling_llama.py:51-297, 452-471
+(EETLlamaSelfMaskedAttention ... EETLlamaForCausalLM), modeling_baichuan.py:
+51-80, 270-317 (ALiBi mask) and pipelines/generation.py:1144-1218 (greedy
+search).  Embedding and lm_head stay fp16 torch ops, as in the reference
+(modeling_llama.py:370-372, 471).
+"""
+import math
+from dataclasses import dataclass
+
+import torch
+
+from . import ops
+
+
+@dataclass
+class DecoderConfig:
+    num_layers: int = 32
+    hidden: int = 4096
+    heads: int = 32
+    d_ff: int = 11008
+    vocab: int = 32000
+    eps: float = 1e-6
+    alibi: bool = False          # False: rotary (LLaMA); True: ALiBi (Baichuan-13B)
+    max_batch: int = 8
+    max_prompt: int = 1024
+    max_full_seq: int = 1153
+
+    @staticmethod
+    def llama_7b(**kw):
+        return DecoderConfig(**kw)
+
+    @staticmethod
+    def baichuan_13b(**kw):
+        d = dict(num_layers=40, hidden=5120, heads=40, d_ff=13696, vocab=64000, alibi=True, max_batch=32,
+                 max_prompt=2048, max_full_seq=2305)
+        d.update(kw)
+        return DecoderConfig(**d)
+
+
+# ---- ALiBi (modeling_baichuan.py:51-80) ------------------------------------
+def alibi_slopes(n):
+    def pow2(n):
+        start = 2 ** (-(2 ** -(math.log2(n) - 3)))
+        return [start * start ** i for i in range(n)]
+    if math.log2(n).is_integer():
+        return pow2(n)
+    c = 2 ** math.floor(math.log2(n))
+    return pow2(c) + alibi_slopes(2 * c)[0::2][: n - c]
+
+
+def alibi_mask(n_head, max_pos, dtype=torch.float16, device="cpu"):
+    """[n_head, max_pos, max_pos]: slope_h * j, -inf above the diagonal; built
+    in fp32 and cast (the `.to(tensor)` at modeling_baichuan.py:273)."""
+    slopes = torch.tensor(alibi_slopes(n_head), dtype=torch.float32)
+    alibi = slopes[:, None, None] * torch.arange(max_pos, dtype=torch.float32)[None, None, :]
+    mask = torch.triu(torch.full((max_pos, max_pos), float("-inf")), 1)
+    return (mask[None] + alibi).to(dtype).to(device)
+
+
+# ---- random-init weights in the reference's state-dict naming ----------------
+def random_state_dict(cfg, seed=1234, quant_mode="ref128"):
+    """Seeded synthetic weights: W ~ N(0, 0.02^2) quantised per output channel,
+    gamma = 1 + 0.1 N(0,1).  Keys follow convert_llama_weights
+    (modeling_llama.py:739-784): 'layer.N.self_attn.qkv_proj.weight' holds the
+    processed int8 [K, N], '.scale' the fp16 scales.  Also returns the
+    unprocessed int8 matrices for checking."""
+    g = torch.Generator().manual_seed(seed)
+    H, F = cfg.hidden, cfg.d_ff
+    sd, raw = {}, {}
+
+    def lin(name, K, N):
+        w = (torch.randn(K, N, generator=g) * 0.02).half()
+        u, p, s = ops.quant_weights(w, torch.int8, True, mode=quant_mode)
+        sd[name + ".weight"], sd[name + ".scale"] = p, s
+        raw[name] = (u, s)
+
+    for i in range(cfg.num_layers):
+        pre = f"layer.{i}."
+        lin(pre + "self_attn.qkv_proj", H, 3 * H)
+        lin(pre + "self_attn.out_proj", H, H)
+        lin(pre + "ffn.intermediate_0", H, F)
+        lin(pre + "ffn.intermediate_1", H, F)
+        lin(pre + "ffn.output", F, H)
+        sd[pre + "self_attn.layernorm.weight"] = (1 + 0.1 * torch.randn(H, generator=g)).half()
+        sd[pre + "ffn.layernorm.weight"] = (1 + 0.1 * torch.randn(H, generator=g)).half()
+    sd["embed_tokens.weight"] = (torch.randn(cfg.vocab, H, generator=g) * 0.02).half()
+    sd["norm.weight"] = (1 + 0.1 * torch.randn(H, generator=g)).half()
+    sd["lm_head.weight"] = (torch.randn(cfg.vocab, H, generator=g) * 0.02).half()
+    return sd, raw
+
+
+class Int8Decoder:
+    """Embedding -> num_layers x (attention op, gated-FFN op) -> final RMSnorm
+    -> lm_head.  Construction order and arguments of the ops are those of
+    EETLlamaSelfMaskedAttention / EETGatedFeedForward (modeling_llama.py:51-146)."""
+
+    def __init__(self, cfg, state_dict, device="cuda:0"):
+        self.cfg = cfg
+        dev = torch.device(device)
+        self.desc = ops.MetaDesc(dtype=torch.float16, batch_size=cfg.max_batch, head_num=cfg.heads,
+                                 hidden_units=cfg.hidden, layer_num=cfg.num_layers, max_seq_len=cfg.max_prompt,
+                                 max_full_seq_len=cfg.max_full_seq, activation_fn="silu", d_kv=0, d_ff=cfg.d_ff,
+                                 cuda_device=str(dev), layernorm_eps=cfg.eps, is_int8=True)
+        e = torch.empty(0)
+        attn_cls = ops.BaichuanMmha if cfg.alibi else ops.LlamaMmha
+        self.layers = []
+        for i in range(cfg.num_layers):
+            pre = f"layer.{i}."
+            t = {k: state_dict[pre + k].to(dev) for k in (
+                "self_attn.qkv_proj.weight", "self_attn.qkv_proj.scale", "self_attn.out_proj.weight",
+                "self_attn.out_proj.scale", "self_attn.layernorm.weight", "ffn.intermediate_0.weight",
+                "ffn.intermediate_0.scale", "ffn.intermediate_1.weight", "ffn.intermediate_1.scale",
+                "ffn.output.weight", "ffn.output.scale", "ffn.layernorm.weight")}
+            attn = attn_cls(self.desc, t["self_attn.qkv_proj.weight"], t["self_attn.qkv_proj.scale"], e, e, e,
+                            t["self_attn.out_proj.weight"], t["self_attn.out_proj.scale"], e,
+                            t["self_attn.layernorm.weight"], e)
+            ffn = ops.GatedFeedForwardNetworkInt8(
+                self.desc, t["ffn.intermediate_0.weight"], t["ffn.intermediate_0.scale"], e,
+                t["ffn.intermediate_1.weight"], t["ffn.intermediate_1.scale"], e, t["ffn.output.weight"],
+                t["ffn.output.scale"], e, t["ffn.layernorm.weight"], e, "decoder_out_cache")
+            self.layers.append((attn, ffn))
+        self.embed = state_dict["embed_tokens.weight"].to(dev)
+        self.norm_w = state_dict["norm.weight"].to(dev)
+        self.final_norm = ops.LayerNorm(self.desc, self.norm_w, e)
+        self.lm_head = state_dict["lm_head.weight"].to(dev)
+        self.pre_padding_len = torch.empty(0, dtype=torch.long)
+        self.reorder_state = torch.empty(0, dtype=torch.long)
+        self.past = 0
+        self._mask = None
+
+    def _alibi(self, first_pass, like):
+        cfg = self.cfg
+        if self._mask is None:
+            # Only rows of the [H, P, P] mask are ever used (row i is slope*j, j <= i),
+            # so the table is kept as [H, P] and expanded on demand.
+            slopes = torch.tensor(alibi_slopes(cfg.heads), dtype=torch.float32)
+            self._mask = (slopes[:, None] * torch.arange(cfg.max_full_seq, dtype=torch.float32)[None, :]
+                          ).to(torch.float16).to(like.device)
+        L = self.past
+        if first_pass:
+            # the op reads the last row of the [H, S, S] mask; hand it that row as a [H, 1->S, S] view
+            return self._mask[:, None, :L].expand(cfg.heads, L, L)
+        return self._mask[:, None, :L].contiguous()
+
+    def __call__(self, input_ids, first_pass=True, attention_mask=None):
+        """modeling_llama.py:262-297 / modeling_baichuan.py:283-333.  Returns the
+        normalised hidden states [B, S, hidden]."""
+        cfg = self.cfg
+        B, S = input_ids.shape
+        assert B <= cfg.max_batch and S <= cfg.max_prompt
+        if attention_mask is None:
+            pad = self.pre_padding_len
+        else:
+            pad = torch.sum(1 - attention_mask, 1, True).to(input_ids.device).long()
+        x = torch.nn.functional.embedding(input_ids, self.embed)
+        bias = torch.empty(0)
+        if cfg.alibi:
+            self.past = S if first_pass else self.past + S
+            bias = self._alibi(first_pass, x)
+        for attn, ffn in self.layers:
+            x = attn.forward(x, pad, self.reorder_state, True, True, first_pass, bias)
+            x = ffn.forward(x, True, True)
+        return self.final_norm.layer_norm(x)
+
+    def logits(self, input_ids, first_pass=True, attention_mask=None):
+        h = self(input_ids, first_pass, attention_mask)
+        return torch.nn.functional.linear(h[:, -1:, :], self.lm_head)
+
+    @torch.no_grad()
+    def greedy(self, input_ids, max_new_tokens, attention_mask=None):
+        """Prefill with the whole prompt, then one token per call: argmax of the
+        last position (generation.py:1144-1218).  Returns [B, max_new_tokens]."""
+        out = []
+        logits = self.logits(input_ids, True, attention_mask)
+        for i in range(max_new_tokens):
+            nxt = torch.argmax(logits[:, -1, :], dim=-1)
+            out.append(nxt)
+            if i + 1 < max_new_tokens:
+                logits = self.logits(nxt[:, None], False, attention_mask)
+        return torch.stack(out, dim=1)

@@ -1,0 +1,463 @@
+"""The reference's operator API (pybind module `EET`, csrc/py11/eet2py.cpp)
+re-hosted on libeet_hip.so through ctypes.
+
+Same names, positional argument order and state machine as the reference ops:
+MetaDesc (eet2py.cpp:26-42), LlamaMmha (:73-86), BaichuanMmha (:58-71),
+GatedFeedForwardNetworkInt8 (:126-134), LayerNorm (:143-145), quant_weights
+(:152-155) and preprocess_weights (:148-150).  The ops of other model families
+are exported as names that raise.
+
+Differences that a caller can observe, all deliberate:
+  * shapes and limits that the reference only `assert`s (compiled out) are
+    checked and raise RuntimeError;
+  * kernels run on torch's current stream, not on a private stream
+    (csrc/op/meta_desc.hpp:58-60);
+  * "processed" int8 weights are in the gfx950 tile layout
+    (eet_pack_gfx950), not the sm80 cutlass layout;
+  * outputs are views of per-process named torch buffers that own their
+    storage (the reference returns from_blob views, llama_mmha.cpp:197-198).
+"""
+import torch
+
+from ._lib import check, lib
+
+_EMPTY = torch.empty(0)
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None and t.numel() > 0 else None
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+# ----------------------------------------------------------------------------
+# named persistent workspaces (the reference's MManager, csrc/op/mmanager.hpp:12-224)
+# ----------------------------------------------------------------------------
+class _Workspaces:
+    def __init__(self):
+        self._bufs = {}
+
+    def get(self, name, numel, dtype, device):
+        key = (name, str(device), dtype)
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < numel:
+            buf = torch.empty(max(int(numel), 1), dtype=dtype, device=device)
+            self._bufs[key] = buf
+        return buf
+
+    def clear(self):
+        self._bufs.clear()
+
+
+workspaces = _Workspaces()
+
+
+# ----------------------------------------------------------------------------
+# MetaDesc
+# ----------------------------------------------------------------------------
+class MetaDesc:
+    """csrc/op/meta_desc.hpp:9-101; constructor keywords as in eet2py.cpp:26-42."""
+
+    def __init__(self, dtype, batch_size, head_num, hidden_units, layer_num, max_seq_len, max_full_seq_len=1,
+                 activation_fn="gelu", d_kv=0, d_ff=0, cuda_device="cuda:0", requires_grad=False,
+                 layernorm_eps=1e-6, is_int8=False):
+        if not isinstance(dtype, torch.dtype):
+            raise TypeError("MetaDesc: dtype must be a torch.dtype")
+        if requires_grad:
+            raise RuntimeError("[EET][ERROR] EET only supports inference (requires_grad must be False)")
+        self.dtype = dtype
+        self.batch_size = int(batch_size)
+        self.head_num = int(head_num)
+        self.hidden_units = int(hidden_units)
+        self.layer_num = int(layer_num)
+        self.max_seq_len = int(max_seq_len)
+        self.max_full_seq_len = int(max_full_seq_len)
+        self.activation_fn = activation_fn
+        self.d_kv = int(d_kv)
+        self.d_ff = int(d_ff)
+        self.device = torch.device(cuda_device)
+        self.layernorm_eps = float(layernorm_eps)
+        self.is_int8 = bool(is_int8)
+
+
+def _require_int8_fp16(desc, who):
+    if desc.dtype != torch.float16 or not desc.is_int8:
+        raise NotImplementedError(
+            f"[EET][ERROR] {who}: only the int8 weight-only path with fp16 activations is implemented "
+            f"(dtype={desc.dtype}, is_int8={desc.is_int8})")
+
+
+def _check_weight(name, w, K, N, device):
+    if w.dtype != torch.int8 or tuple(w.shape) != (K, N) or not w.is_contiguous():
+        raise RuntimeError(f"[EET][ERROR] {name}: expected contiguous int8 [{K}, {N}], got {w.dtype} {tuple(w.shape)}")
+    if w.device.type != "cuda":
+        raise RuntimeError(f"[EET][ERROR] {name}: weight must be on the GPU")
+
+
+def _check_vec(name, v, N):
+    if v.dtype != torch.float16 or v.numel() != N or not v.is_contiguous() or v.device.type != "cuda":
+        raise RuntimeError(f"[EET][ERROR] {name}: expected contiguous fp16 GPU tensor of {N} elements, "
+                           f"got {v.dtype} {tuple(v.shape)} on {v.device}")
+
+
+def _gemm(a, w, scale, out, M, N, K):
+    check(lib().eet_gemm_w8a16(a.data_ptr(), w.data_ptr(), scale.data_ptr(), out.data_ptr(), M, N, K, None, 0,
+                               _stream()), "eet_gemm_w8a16")
+
+
+def _rmsnorm(x, gamma, out, M, N, eps):
+    check(lib().eet_rmsnorm(x.data_ptr(), gamma.data_ptr(), out.data_ptr(), M, N, eps, _stream()), "eet_rmsnorm")
+
+
+# ----------------------------------------------------------------------------
+# attention ops
+# ----------------------------------------------------------------------------
+class _MmhaInt8:
+    """Shared body of LlamaMmha (rotary) and BaichuanMmha (ALiBi)."""
+
+    _rope = True
+    _name = "LlamaMmha"
+
+    def __init__(self, desc, QKV_weights, QKV_scale, Q_bias, K_bias, V_bias, Output_weights, Output_scale,
+                 Output_bias, layernorm_weights, layernorm_bias):
+        _require_int8_fp16(desc, self._name)
+        for nm, b in (("Q_bias", Q_bias), ("K_bias", K_bias), ("V_bias", V_bias), ("Output_bias", Output_bias),
+                      ("layernorm_bias", layernorm_bias)):
+            if b is not None and b.numel() != 0:
+                raise NotImplementedError(f"[EET][ERROR] {self._name}: {nm} is not supported on the int8 path "
+                                          "(LLaMA / Baichuan have none)")
+        self.desc = desc
+        H = desc.head_num
+        if desc.d_kv == 0:
+            self.dh, self.inner = desc.hidden_units // H, desc.hidden_units
+        else:
+            self.dh, self.inner = desc.d_kv, desc.d_kv * H
+        if self.dh not in (32, 64, 128):
+            raise RuntimeError(f"[EET][ERROR] {self._name}: head size {self.dh} not supported (32, 64, 128)")
+        hidden = desc.hidden_units
+        _check_weight("QKV_weights", QKV_weights, hidden, 3 * self.inner, desc.device)
+        _check_weight("Output_weights", Output_weights, self.inner, hidden, desc.device)
+        _check_vec("QKV_scale", QKV_scale, 3 * self.inner)
+        _check_vec("Output_scale", Output_scale, hidden)
+        _check_vec("layernorm_weights", layernorm_weights, hidden)
+        # keep the tensors alive: the kernels read them through raw pointers
+        self.qkv_w, self.qkv_s, self.o_w, self.o_s, self.gamma = (QKV_weights, QKV_scale, Output_weights,
+                                                                  Output_scale, layernorm_weights)
+        dev = QKV_weights.device
+        self.t_cap = desc.max_full_seq_len
+        # KV cache, private to the op (csrc/op/llama_mmha.cpp:47-48); layout [B][H][T][dh]
+        self.k_cache = torch.zeros(desc.batch_size, H, self.t_cap, self.dh, dtype=torch.float16, device=dev)
+        self.v_cache = torch.zeros_like(self.k_cache)
+        self.step = 1
+        self.first_batch = 0
+
+    def forward(self, input, pre_padding_len, reorder_state, pre_layernorm, add_residual, first_pass,
+                relative_attention_bias=_EMPTY):
+        # pre_layernorm / add_residual are accepted and ignored exactly as in the
+        # reference: it always normalises first and always adds the input back
+        # (csrc/op/llama_mmha.cpp:136, 222, 462).
+        desc, H, dh = self.desc, self.desc.head_num, self.dh
+        if input.dtype != torch.float16 or input.dim() != 3 or input.shape[2] != desc.hidden_units:
+            raise RuntimeError(f"[EET][ERROR] {self._name}: input must be fp16 [B, S, {desc.hidden_units}], got "
+                               f"{input.dtype} {tuple(input.shape)}")
+        if input.device.type != "cuda":
+            raise RuntimeError(f"[EET][ERROR] {self._name}: input must be on the GPU")
+        if reorder_state is not None and reorder_state.numel() != 0:
+            raise NotImplementedError(f"[EET][ERROR] {self._name}: beam-search cache reorder is not implemented")
+        x = input.contiguous()
+        B, S, hidden = x.shape
+        if B > desc.batch_size:
+            raise RuntimeError(f"[EET][ERROR] {self._name}: batch {B} exceeds batch_size {desc.batch_size}")
+        dev = x.device
+        pad = pre_padding_len if (pre_padding_len is not None and pre_padding_len.numel() != 0) else None
+        if pad is not None:
+            if pad.dtype != torch.int64 or pad.numel() < B or pad.device.type != "cuda":
+                raise RuntimeError(f"[EET][ERROR] {self._name}: pre_padding_len must be an int64 GPU tensor of B elements")
+            pad = pad.contiguous()
+        bias = relative_attention_bias if (relative_attention_bias is not None
+                                           and relative_attention_bias.numel() != 0) else None
+        if self._rope and bias is not None:
+            raise RuntimeError(f"[EET][ERROR] {self._name}: relative_attention_bias is not used by the rotary op")
+        if first_pass:
+            if S > desc.max_seq_len or S > self.t_cap:
+                raise RuntimeError(f"[EET][ERROR] {self._name}: prompt length {S} exceeds max_seq_len "
+                                   f"{desc.max_seq_len} / max_full_seq_len {self.t_cap}")
+            self.step, self.first_batch = S, B
+            t0, time_step = 0, -1
+        else:
+            if S != 1:
+                raise RuntimeError(f"[EET][ERROR] {self._name}: incremental call needs seq_len 1, got {S}")
+            if self.step + 1 > self.t_cap:
+                raise RuntimeError(f"[EET][ERROR] {self._name}: step {self.step + 1} exceeds max_full_seq_len "
+                                   f"{self.t_cap}")
+            self.step += 1
+            t0, time_step = self.step - 1, self.step - 1
+        M = B * S
+        L = lib()
+        f16 = torch.float16
+        xn = workspaces.get("layernorm", desc.batch_size * max(desc.max_seq_len, 1) * hidden, f16, dev)
+        qkv = workspaces.get("qkv", desc.batch_size * max(desc.max_seq_len, 1) * 3 * self.inner, f16, dev)
+        qbuf = workspaces.get("q_buf", desc.batch_size * max(desc.max_seq_len, 1) * self.inner, f16, dev)
+        cbuf = workspaces.get("context_buf", desc.batch_size * max(desc.max_seq_len, 1) * self.inner, f16, dev)
+        out = workspaces.get("self_mask_attn_cache", desc.batch_size * max(desc.max_seq_len, 1) * hidden, f16, dev)
+        _rmsnorm(x, self.gamma, xn, M, hidden, desc.layernorm_eps)
+        _gemm(xn, self.qkv_w, self.qkv_s, qkv, M, 3 * self.inner, hidden)
+        check(L.eet_qkv_split(qkv.data_ptr(), qbuf.data_ptr(), self.k_cache.data_ptr(), self.v_cache.data_ptr(),
+                              B, S, H, dh, 1 if self._rope else 0, time_step, t0, self.t_cap, _stream()),
+              "eet_qkv_split")
+        if first_pass:
+            alibi = None
+            if bias is not None:
+                # [H, S, S] mask whose row i holds slope*j for j <= i: its last row is the whole table
+                if bias.dim() != 3 or bias.shape[0] != H or bias.shape[2] != S:
+                    raise RuntimeError(f"[EET][ERROR] {self._name}: relative_attention_bias must be [H, S, S]")
+                alibi = bias[:, -1, :].to(f16).contiguous()
+            check(L.eet_prefill_attention(qbuf.data_ptr(), self.k_cache.data_ptr(), self.v_cache.data_ptr(),
+                                          cbuf.data_ptr(), _ptr(alibi), _ptr(pad), B, H, S, dh, self.t_cap,
+                                          _stream()), "eet_prefill_attention")
+        else:
+            alibi = None
+            if bias is not None:
+                if bias.numel() != H * self.step:
+                    raise RuntimeError(f"[EET][ERROR] {self._name}: relative_attention_bias must be [H, 1, step] "
+                                       f"with step={self.step}, got {tuple(bias.shape)}")
+                alibi = bias.to(f16).contiguous()
+            need = L.eet_mmha_decode_workspace(B, H, dh, self.step)
+            ws = workspaces.get("mmha_ws", max(need // 4, 1), torch.float32, dev)
+            # k, v already sit in the cache (written by eet_qkv_split), so no append here
+            check(L.eet_mmha_decode(qbuf.data_ptr(), None, None, 0, self.k_cache.data_ptr(),
+                                    self.v_cache.data_ptr(), cbuf.data_ptr(), _ptr(alibi), _ptr(pad), B, H, dh,
+                                    self.step, self.t_cap, ws.data_ptr(), ws.numel() * 4, _stream()),
+                  "eet_mmha_decode")
+        _gemm(cbuf, self.o_w, self.o_s, out, M, hidden, self.inner)
+        check(L.eet_residual_add(out.data_ptr(), x.data_ptr(), M, hidden, _stream()), "eet_residual_add")
+        self._keep = (x, pad, alibi)  # inputs of kernels still in flight
+        return out[: M * hidden].view(B, S, hidden)
+
+
+class LlamaMmha(_MmhaInt8):
+    """csrc/op/llama_mmha.cpp:14-266."""
+    _rope = True
+    _name = "LlamaMmha"
+
+
+class BaichuanMmha(_MmhaInt8):
+    """csrc/op/baichuan_mmha.cpp:81-216: no rotary; an ALiBi tensor is passed in
+    ([H, S, S] for the prompt, [H, 1, step] per decode step)."""
+    _rope = False
+    _name = "BaichuanMmha"
+
+
+# ----------------------------------------------------------------------------
+# gated FFN
+# ----------------------------------------------------------------------------
+class GatedFeedForwardNetworkInt8:
+    """csrc/op/gated_ffn_int8.cpp:12-132, 328-357."""
+
+    def __init__(self, desc, Intermediate_0_weights, Intermediate_0_scale, Intermediate_0_bias,
+                 Intermediate_1_weights, Intermediate_1_scale, Intermediate_1_bias, Output_weights, Output_scale,
+                 Output_bias, layernorm_weights, layernorm_bias, ffn_cache_name="out_cache"):
+        _require_int8_fp16(desc, "GatedFeedForwardNetworkInt8")
+        if desc.activation_fn != "silu":
+            # the reference prints "unsupported activation" and goes on (gated_ffn_int8.cpp:57-61)
+            raise NotImplementedError(f"[EET][ERROR] GatedFeedForwardNetworkInt8: activation "
+                                      f"'{desc.activation_fn}' is not implemented (silu only)")
+        for nm, b in (("Intermediate_0_bias", Intermediate_0_bias), ("Intermediate_1_bias", Intermediate_1_bias),
+                      ("Output_bias", Output_bias), ("layernorm_bias", layernorm_bias)):
+            if b is not None and b.numel() != 0:
+                raise NotImplementedError(f"[EET][ERROR] GatedFeedForwardNetworkInt8: {nm} is not supported")
+        self.desc = desc
+        hidden = desc.hidden_units
+        self.d_ff = desc.d_ff if desc.d_ff != 0 else 4 * hidden  # gated_ffn_int8.cpp:62-68
+        dev = desc.device
+        _check_weight("Intermediate_0_weights", Intermediate_0_weights, hidden, self.d_ff, dev)
+        _check_weight("Intermediate_1_weights", Intermediate_1_weights, hidden, self.d_ff, dev)
+        _check_weight("Output_weights", Output_weights, self.d_ff, hidden, dev)
+        _check_vec("Intermediate_0_scale", Intermediate_0_scale, self.d_ff)
+        _check_vec("Intermediate_1_scale", Intermediate_1_scale, self.d_ff)
+        _check_vec("Output_scale", Output_scale, hidden)
+        _check_vec("layernorm_weights", layernorm_weights, hidden)
+        self.w0, self.s0, self.w1, self.s1, self.w2, self.s2, self.gamma = (
+            Intermediate_0_weights, Intermediate_0_scale, Intermediate_1_weights, Intermediate_1_scale,
+            Output_weights, Output_scale, layernorm_weights)
+        self.cache_name = ffn_cache_name
+
+    def forward(self, input, pre_layernorm, add_residual):
+        desc = self.desc
+        if input.dtype != torch.float16 or input.dim() != 3 or input.shape[2] != desc.hidden_units:
+            raise RuntimeError(f"[EET][ERROR] GatedFeedForwardNetworkInt8: input must be fp16 [B, S, "
+                               f"{desc.hidden_units}], got {input.dtype} {tuple(input.shape)}")
+        if add_residual and not pre_layernorm:
+            raise NotImplementedError("[EET][ERROR] GatedFeedForwardNetworkInt8: post-layernorm mode is not implemented")
+        x = input.contiguous()
+        B, S, hidden = x.shape
+        if B > desc.batch_size or S > max(desc.max_seq_len, 1):
+            raise RuntimeError(f"[EET][ERROR] GatedFeedForwardNetworkInt8: input [{B}, {S}] exceeds "
+                               f"[{desc.batch_size}, {desc.max_seq_len}]")
+        M, dev, f16 = B * S, x.device, torch.float16
+        cap = desc.batch_size * max(desc.max_seq_len, 1)
+        xn = workspaces.get("layernorm_tensor", cap * hidden, f16, dev)
+        act = workspaces.get("ffn_inner_act", cap * self.d_ff, f16, dev)
+        lin = workspaces.get("ffn_inner_linear", cap * self.d_ff, f16, dev)
+        out = workspaces.get(self.cache_name, cap * hidden, f16, dev)
+        L = lib()
+        _rmsnorm(x, self.gamma, xn, M, hidden, desc.layernorm_eps)
+        _gemm(xn, self.w0, self.s0, act, M, self.d_ff, hidden)
+        _gemm(xn, self.w1, self.s1, lin, M, self.d_ff, hidden)
+        check(L.eet_swiglu(act.data_ptr(), lin.data_ptr(), M, self.d_ff, _stream()), "eet_swiglu")
+        _gemm(act, self.w2, self.s2, out, M, hidden, self.d_ff)
+        if add_residual:
+            check(L.eet_residual_add(out.data_ptr(), x.data_ptr(), M, hidden, _stream()), "eet_residual_add")
+        self._keep = x
+        return out[: M * hidden].view(B, S, hidden)
+
+
+class LayerNorm:
+    """csrc/op/layer_norm.cpp:8-33: RMSnorm when beta is empty."""
+
+    def __init__(self, desc, gamma, beta):
+        if desc.dtype != torch.float16:
+            raise NotImplementedError("[EET][ERROR] LayerNorm: fp16 only")
+        if beta is not None and beta.numel() != 0:
+            raise NotImplementedError("[EET][ERROR] LayerNorm: only the RMSnorm form (empty beta) is implemented")
+        _check_vec("gamma", gamma, desc.hidden_units)
+        self.desc, self.gamma = desc, gamma
+        self.output = torch.zeros(desc.batch_size, max(desc.max_seq_len, 1), desc.hidden_units,
+                                  dtype=torch.float16, device=gamma.device)
+
+    def layer_norm(self, input):
+        desc = self.desc
+        if input.dtype != torch.float16 or input.dim() != 3 or input.shape[2] != desc.hidden_units:
+            raise RuntimeError("[EET][ERROR] LayerNorm: input must be fp16 [B, S, hidden]")
+        x = input.contiguous()
+        B, S, hidden = x.shape
+        if B * S > self.output.shape[0] * self.output.shape[1]:
+            raise RuntimeError("[EET][ERROR] LayerNorm: input larger than batch_size * max_seq_len")
+        _rmsnorm(x, self.gamma, self.output, B * S, hidden, desc.layernorm_eps)
+        self._keep = x
+        return self.output.view(-1)[: B * S * hidden].view(B, S, hidden)
+
+
+# ----------------------------------------------------------------------------
+# offline packer
+# ----------------------------------------------------------------------------
+def _quantize(weight, mode):
+    K, N = weight.shape
+    q = torch.empty(K, N, dtype=torch.int8)
+    scale = torch.empty(N, dtype=weight.dtype)
+    dt = 0 if weight.dtype == torch.float32 else 1
+    check(lib().eet_quantize_int8(weight.data_ptr(), dt, K, N, mode, q.data_ptr(), scale.data_ptr()),
+          "eet_quantize_int8")
+    return q, scale
+
+
+def pack_weights(q):
+    """int8 [K, N] row-major -> gfx950 tile layout (same shape and byte count)."""
+    if q.device.type != "cpu" or q.dtype != torch.int8 or q.dim() != 2 or not q.is_contiguous():
+        raise RuntimeError("[EET][ERROR] pack_weights: expected a contiguous CPU int8 [K, N] tensor")
+    out = torch.empty_like(q)
+    check(lib().eet_pack_gfx950(q.data_ptr(), q.shape[0], q.shape[1], out.data_ptr()), "eet_pack_gfx950")
+    return out
+
+
+def unpack_weights(p):
+    if p.device.type != "cpu" or p.dtype != torch.int8 or p.dim() != 2 or not p.is_contiguous():
+        raise RuntimeError("[EET][ERROR] unpack_weights: expected a contiguous CPU int8 [K, N] tensor")
+    out = torch.empty_like(p)
+    check(lib().eet_unpack_gfx950(p.data_ptr(), p.shape[0], p.shape[1], out.data_ptr()), "eet_unpack_gfx950")
+    return out
+
+
+def pack_weights_torch(q):
+    """eet_pack_gfx950 expressed as torch view / permute ops, so that a weight
+    that already lives on the GPU can be packed there.  Same result, any device."""
+    if q.dtype != torch.int8 or q.dim() != 2 or q.shape[0] % 64 or q.shape[1] % 16:
+        raise RuntimeError("[EET][ERROR] pack_weights_torch: expected int8 [K, N] with K % 64 == 0 and N % 16 == 0")
+    K, N = q.shape
+    t = (q.view(torch.uint8) ^ 0x80).view(K // 64, 4, 16, N // 16, 16)   # [kt, g, b, nt, i]
+    return t.permute(3, 0, 1, 4, 2).contiguous().view(torch.int8).view(K, N)
+
+
+def quant_weights_torch(w, mode="ref128"):
+    """The quantiser as torch ops on w's device (fp32 math, same rules as
+    eet_quantize_int8): returns (unprocessed int8 [K, N], scales in w's dtype)."""
+    w32 = w.float()
+    amax = w32.abs().amax(0)
+    if mode == "ref128":
+        s32 = amax * (1.0 / 128.0)
+        r = w32 / s32
+        r = torch.where(r >= 0, torch.floor(r.abs() + 0.5), -torch.floor(r.abs() + 0.5))
+        r = torch.where(torch.isnan(r), torch.full_like(r, 127.0), r).clamp(-128, 127)
+    else:
+        s32 = amax / 127.0
+        r = w32 / s32
+        r = torch.where(r >= 0, torch.floor(r.abs() + 0.5), -torch.floor(r.abs() + 0.5))
+        r = torch.where(torch.isnan(r), torch.zeros_like(r), r).clamp(-127, 127)
+    return r.to(torch.int8), s32.to(w.dtype)
+
+
+def quant_weights(origin_weight, quant_type, return_unprocessed_quantized_tensor=False, mode="ref128"):
+    """symmetric_quantize_last_axis_of_tensor
+    (3rdparty/cutlass_kernels/fpA_intB_gemm_wrapper.cu:26-105).  Returns
+    [processed, scales] or [unprocessed, processed, scales]; `processed` is the
+    gfx950 layout.  mode="sym127" selects the /127 generator (not a reference mode)."""
+    w = origin_weight
+    if w.device.type != "cpu":
+        raise RuntimeError("weight must be a CPU tensor")
+    if not w.is_contiguous():
+        raise RuntimeError("weight must be contiguous")
+    if w.numel() == 0:
+        raise RuntimeError("weight should not be empty tensor")
+    if w.dim() not in (2, 3):
+        raise RuntimeError("Invalid dim. The dim of weight should be 2 or 3")
+    if w.dtype not in (torch.float32, torch.float16):
+        raise RuntimeError("Invalid datatype. Weight must be FP16 or FP32")
+    if quant_type == torch.quint4x2:
+        raise NotImplementedError("[EET][ERROR] quant_weights: int4 quantisation is not implemented")
+    if quant_type != torch.int8:
+        raise RuntimeError("Must be int4 or int8 quantization")
+    m = {"ref128": 0, "sym127": 1}[mode]
+    mats = [w] if w.dim() == 2 else list(w.unbind(0))
+    qs, ps, ss = [], [], []
+    for mat in mats:
+        q, s = _quantize(mat.contiguous(), m)
+        qs.append(q)
+        ps.append(pack_weights(q))
+        ss.append(s)
+    if w.dim() == 2:
+        unprocessed, processed, scales = qs[0], ps[0], ss[0]
+    else:
+        unprocessed, processed, scales = torch.stack(qs), torch.stack(ps), torch.stack(ss)
+    if return_unprocessed_quantized_tensor:
+        return [unprocessed, processed, scales]
+    return [processed, scales]
+
+
+def preprocess_weights(origin_weight, is_int4=False):
+    """preprocess_weights_cuda (fpA_intB_gemm_wrapper.cu:107-126): row-major
+    int8 [K, N] -> the layout the GEMM reads."""
+    if is_int4:
+        raise NotImplementedError("[EET][ERROR] preprocess_weights: int4 is not implemented")
+    if origin_weight.device.type != "cpu":
+        raise RuntimeError("origin_weight must be a CPU tensor")
+    return pack_weights(origin_weight.contiguous())
+
+
+def _not_on_this_path(name):
+    class _Stub:
+        def __init__(self, *a, **k):
+            raise NotImplementedError(f"[EET][ERROR] {name} is not part of the int8 weight-only path "
+                                      "implemented by this library")
+    _Stub.__name__ = name
+    return _Stub
+
+
+# names the reference's Python imports from `EET` but that belong to other model families
+GatedFeedForwardNetwork = _not_on_this_path("GatedFeedForwardNetwork")
+FeedForwardNetwork = _not_on_this_path("FeedForwardNetwork")
+MultiHeadAttention = _not_on_this_path("MultiHeadAttention")
+CrossMultiHeadAttention = _not_on_this_path("CrossMultiHeadAttention")
+MaskedMultiHeadAttention = _not_on_this_path("MaskedMultiHeadAttention")
+Embedding = _not_on_this_path("Embedding")

@@ -1,0 +1,151 @@
+/*
+ * eet_hip.h -- C ABI of libeet_hip.so: the MI355X (gfx950) implementation of
+ * EET's int8 weight-only linear path and the decode attention beside it.
+ *
+ * This is the boundary a maintainer of the reference binds in place of the
+ * pybind11 module `EET` (csrc/py11/eet2py.cpp) and the kernels under csrc/op,
+ * csrc/core and 3rdparty/cutlass_kernels that it reaches.  Plain pointers and
+ * sizes only; no torch types, no C++ exceptions cross it.
+ *
+ * Conventions
+ *   - every function returns 0 on success and a negative eet_status on failure;
+ *     eet_last_error() then returns a thread-local, human-readable message
+ *     (the reference throws std::runtime_error: csrc/op/common.hpp:55-64,
+ *     3rdparty/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm_template.h:156-176).
+ *   - "half" buffers are IEEE binary16, passed as void*.
+ *   - device functions enqueue on `stream` (a hipStream_t passed as void*;
+ *     NULL = the legacy default stream) and return without synchronising.  The
+ *     reference used one private stream (csrc/op/meta_desc.hpp:58-60); here the
+ *     caller supplies its own.
+ *   - weights are [K = in_features, N = out_features] (the reference's
+ *     convention, python/eet/transformers/modeling_llama.py:764-766).
+ */
+#ifndef EET_HIP_H
+#define EET_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum eet_status {
+    EET_OK = 0,
+    EET_ERR_INVALID_ARGUMENT = -1, /* null pointer, negative size, bad enum */
+    EET_ERR_UNSUPPORTED_SHAPE = -2, /* shape the kernels cannot take (e.g. K % 64 != 0) */
+    EET_ERR_HIP = -3,               /* a HIP runtime call failed */
+    EET_ERR_WORKSPACE = -4          /* workspace missing or too small */
+} eet_status;
+
+enum { EET_DTYPE_F32 = 0, EET_DTYPE_F16 = 1 };
+enum { EET_QUANT_REF128 = 0, EET_QUANT_SYM127 = 1 };
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char *eet_last_error(void);
+
+/* Version tag of the packed weight layout produced by eet_pack_gfx950. */
+int eet_packed_layout_version(void);
+
+/* ------------------------------------------------------------------------
+ * Offline weight packer (host CPU, no GPU needed).
+ * ---------------------------------------------------------------------- */
+
+/* Per-output-channel symmetric int8 quantisation of w[K][N] (row-major,
+ * w_dtype = EET_DTYPE_F32 or EET_DTYPE_F16).  Writes q[K][N] (row-major,
+ * "unprocessed") and scale[N] in w's dtype.
+ *   EET_QUANT_REF128: bit-exact with the reference quantiser: scale =
+ *     absmax / 128, q = clamp(round(w / scale_fp32), -128, 127).
+ *   EET_QUANT_SYM127: scale = absmax / 127, q in [-127, 127]; zero column -> 0.
+ * Replaces ft::symmetric_quantize, int8 branch
+ * (3rdparty/cutlass_kernels/cutlass_preprocessors.cc:581-678), reached from
+ * symmetric_quantize_last_axis_of_tensor
+ * (3rdparty/cutlass_kernels/fpA_intB_gemm_wrapper.cu:26-105). */
+int eet_quantize_int8(const void *w, int w_dtype, size_t K, size_t N, int mode,
+                      int8_t *q, void *scale);
+
+/* Permute q[K][N] into the gfx950 tile-interleaved layout the GEMM kernels
+ * read (K % 64 == 0, N % 16 == 0; same byte count).  Replaces
+ * preprocess_weights_for_mixed_gemm (cutlass_preprocessors.cc:497-534), whose
+ * sm75/sm80 layout has no meaning on gfx950.  eet_unpack_gfx950 is the inverse. */
+int eet_pack_gfx950(const int8_t *q, size_t K, size_t N, int8_t *packed);
+int eet_unpack_gfx950(const int8_t *packed, size_t K, size_t N, int8_t *q);
+
+/* The reference's own processed layout for sm75..sm89 and its inverse, so that
+ * int8 state dicts saved by the reference (cutlass_preprocessors.cc:497-534;
+ * K % 64 == 0 and N % 64 == 0) can be re-packed for gfx950. */
+int eet_preprocess_ref_sm80(const int8_t *q, size_t K, size_t N, int8_t *processed);
+int eet_unprocess_ref_sm80(const int8_t *processed, size_t K, size_t N, int8_t *q);
+
+/* ------------------------------------------------------------------------
+ * Device kernels (gfx950).
+ * ---------------------------------------------------------------------- */
+
+/* C[M][N] (half) = A[M][K] (half) . (int8 W[K][N] * scale[N] (half)), fp32
+ * accumulation, one rounding to half.  Wpacked comes from eet_pack_gfx950.
+ * M <= 32 takes the HBM-streaming small-M kernel, larger M the LDS-staged MFMA
+ * kernel.  No workspace is needed (NULL / 0 accepted).
+ * Replaces fastertransformer::gemm_fp16_int_bias_act<uint8_t>
+ * (3rdparty/cutlass_kernels/fpA_intB_gemm.cu:35-62) as called with
+ * bias = nullptr and no activation from csrc/op/llama_mmha.cpp:313-337,
+ * 428-447 and csrc/op/gated_ffn_int8.cpp:253-326. */
+int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *scale, void *C,
+                   int M, int N, int K, void *workspace, size_t workspace_bytes,
+                   void *stream);
+
+/* Masked multi-head decode attention for one new token per sequence.
+ *   q, k, v   [B][H][dh] half; with qkv_stride != 0 they are rows of a fused
+ *             buffer: element (b, h, d) at base[b * qkv_stride + h * dh + d]
+ *   k_cache, v_cache  [B_cap][H][T_cap][dh] half; the new k, v are appended at
+ *             row step-1, rows [0, step) are attended
+ *   alibi     NULL or [H][step] half, added to the scaled logits
+ *   pad       NULL or [B] int64: rows t < pad[b] get zero weight
+ *   ctx       [B][H*dh] half
+ *   workspace eet_mmha_decode_workspace(B, H, dh, step) bytes of device memory
+ * softmax denominator carries the reference's + 1e-6.
+ * Replaces masked_attention_dispatch (csrc/core/attention_dispatch.cu:888-928)
+ * and fused_masked_attention_dispatch with q_bias == nullptr (:1338-1426). */
+size_t eet_mmha_decode_workspace(int B, int H, int dh, int step);
+int eet_mmha_decode(const void *q, const void *k, const void *v, long qkv_stride,
+                    void *k_cache, void *v_cache, void *ctx, const void *alibi,
+                    const int64_t *pad, int B, int H, int dh, int step, int T_cap,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+/* out[M][N] = x * rsqrt(mean(x^2) + eps) * gamma.  Replaces RMSnorm
+ * (csrc/core/layer_norm.cu:580-625). */
+int eet_rmsnorm(const void *x, const void *gamma, void *out, int M, int N, float eps,
+                void *stream);
+
+/* Split a fused qkv[B][S][3][H][dh] row.  With rope != 0, q and k are rotated
+ * NeoX-style (pairs i, i + dh/2) at position s (time_step < 0) or time_step.
+ *   q_out  [B][H][S][dh]
+ *   k and v go straight into the caches [B_cap][H][T_cap][dh] at rows
+ *   t0 + s (t0 = 0 for prefill, step-1 for decode).
+ * Replaces fused_QKV_bias_rotary_kernel / fused_QKV_transpose
+ * (csrc/core/self_add_bias.cu:442-487, 303-360) plus copyKV_transpose
+ * (csrc/core/transpose.cu:116-124). */
+int eet_qkv_split(const void *qkv, void *q_out, void *k_cache, void *v_cache, int B, int S,
+                  int H, int dh, int rope, int time_step, int t0, int T_cap, void *stream);
+
+/* gate[M][N] = up * gate / (1 + exp(-gate)).  Replaces gated_act_kernel, silu
+ * (csrc/core/activation_kernel.cu:275-338). */
+int eet_swiglu(void *gate, const void *up, int M, int N, void *stream);
+
+/* out[M][N] += residual[M][N].  Replaces add_bias_input_kernel with
+ * bias == nullptr (csrc/core/add_bias.cu:51-73). */
+int eet_residual_add(void *out, const void *residual, int M, int N, void *stream);
+
+/* Causal prefill attention over the prompt, reading K and V from the caches
+ * filled by eet_qkv_split.  q [B][H][S][dh]; ctx [B][S][H*dh]; alibi NULL or
+ * [H][S] half (slope * j, the diagonal row of the reference's mask); pad as in
+ * eet_mmha_decode (padded query rows give zeros).  Replaces the unfused
+ * QK^T / softmax / PV / transpose sequence of csrc/op/llama_mmha.cpp:160-186
+ * and csrc/op/baichuan_mmha.cpp:120-150. */
+int eet_prefill_attention(const void *q, const void *k_cache, const void *v_cache, void *ctx,
+                          const void *alibi, const int64_t *pad, int B, int H, int S, int dh,
+                          int T_cap, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EET_HIP_H */

@@ -1,0 +1,111 @@
+"""The C-ABI library: loads without a GPU, exports exactly what include/eet_hip.h
+declares, and validates arguments before touching the device."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from eet_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "eet_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(eet_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    syms = declared_symbols()
+    assert len(syms) >= 14
+    assert sorted(_lib.SIGNATURES) == syms
+
+
+def test_library_exports_every_declared_symbol():
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for s in declared_symbols():
+        assert hasattr(handle, s), s
+
+
+def test_layout_version_and_last_error():
+    L = _lib.lib()
+    assert L.eet_packed_layout_version() == 1
+    rc = L.eet_pack_gfx950(None, 64, 16, None)
+    assert rc == -1 and b"null pointer" in L.eet_last_error()
+
+
+def test_quantize_argument_errors():
+    L = _lib.lib()
+    w = np.zeros((4, 4), np.float32)
+    q = np.zeros((4, 4), np.int8)
+    s = np.zeros(4, np.float32)
+    assert L.eet_quantize_int8(w.ctypes.data, 7, 4, 4, 0, q.ctypes.data, s.ctypes.data) == -1
+    assert L.eet_quantize_int8(w.ctypes.data, 0, 4, 4, 9, q.ctypes.data, s.ctypes.data) == -1
+    assert L.eet_quantize_int8(None, 0, 4, 4, 0, q.ctypes.data, s.ctypes.data) == -1
+    assert L.eet_quantize_int8(w.ctypes.data, 0, 4, 4, 0, q.ctypes.data, s.ctypes.data) == 0
+
+
+def test_device_entry_points_validate_before_launch():
+    """Bad arguments are refused on the host: no GPU is needed to see the error."""
+    L = _lib.lib()
+    buf = np.zeros(4096, np.uint8)
+    p = buf.ctypes.data
+    assert L.eet_gemm_w8a16(None, p, p, p, 1, 16, 64, None, 0, None) == -1
+    assert L.eet_gemm_w8a16(p, p, p, p, 1, 16, 100, None, 0, None) == -2      # K % 64
+    assert L.eet_gemm_w8a16(p, p, p, p, 1, 24, 64, None, 0, None) == -2       # N % 16
+    assert b"K % 64" in L.eet_last_error()
+    assert L.eet_gemm_w8a16(p, p, p, p, 0, 16, 64, None, 0, None) == 0        # empty batch: nothing to do
+    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 128, 9, 8, None, 0, None) == -1  # step > cap
+    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 96, 1, 8, None, 0, None) == -2   # head size
+    assert L.eet_mmha_decode(p, p, None, 0, p, p, p, None, None, 1, 1, 128, 1, 8, None, 0, None) == -1     # k without v
+    need = L.eet_mmha_decode_workspace(8, 32, 128, 1100)
+    assert need > 0
+    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 8, 32, 128, 1100, 1153, None, 0, None) == -4
+    assert L.eet_rmsnorm(p, p, p, 1, 20000, 1e-6, None) == -2
+    assert L.eet_qkv_split(p, p, p, p, 1, 4, 1, 128, 1, -1, 6, 8, None) == -1  # rows past the cache end
+    assert L.eet_swiglu(p, p, 1, 12, None) == -2
+    assert L.eet_residual_add(p, None, 1, 16, None) == -1
+    assert L.eet_prefill_attention(p, p, p, p, None, None, 1, 1, 4096, 128, 4096, None) == -2
+
+
+def test_python_api_errors():
+    import eet_amd
+    with pytest.raises(RuntimeError, match="contiguous"):
+        eet_amd.quant_weights(torch.zeros(64, 32).t(), torch.int8)
+    with pytest.raises(RuntimeError, match="dim"):
+        eet_amd.quant_weights(torch.zeros(64), torch.int8)
+    with pytest.raises(RuntimeError, match="FP16 or FP32"):
+        eet_amd.quant_weights(torch.zeros(64, 16, dtype=torch.float64), torch.int8)
+    with pytest.raises(RuntimeError, match="empty"):
+        eet_amd.quant_weights(torch.zeros(0, 16), torch.int8)
+    with pytest.raises(RuntimeError, match="int4 or int8"):
+        eet_amd.quant_weights(torch.zeros(64, 16), torch.int32)
+    with pytest.raises(NotImplementedError):
+        eet_amd.quant_weights(torch.zeros(64, 16), torch.quint4x2)
+    p, s = eet_amd.quant_weights(torch.ones(64, 16), torch.int8)
+    assert p.dtype == torch.int8 and p.shape == (64, 16) and s.dtype == torch.float32 and s.shape == (16,)
+    u, p, s = eet_amd.quant_weights(torch.ones(2, 64, 16).half(), torch.int8, True)
+    assert u.shape == (2, 64, 16) and s.shape == (2, 16) and s.dtype == torch.float16
+    with pytest.raises(NotImplementedError):
+        eet_amd.MultiHeadAttention()
+    import EET
+    for name in ("MetaDesc", "LlamaMmha", "BaichuanMmha", "GatedFeedForwardNetworkInt8", "GatedFeedForwardNetwork",
+                 "Embedding", "preprocess_weights", "quant_weights", "FeedForwardNetwork", "MultiHeadAttention",
+                 "CrossMultiHeadAttention", "MaskedMultiHeadAttention", "LayerNorm"):
+        assert hasattr(EET, name)
+    d = EET.MetaDesc(torch.float16, 8, 32, 4096, 32, 1024, 1153, "silu", 0, 11008, "cuda:0", False, 1e-6, True)
+    assert d.max_full_seq_len == 1153 and d.d_ff == 11008 and d.is_int8
+    with pytest.raises(NotImplementedError):
+        EET.LlamaMmha(EET.MetaDesc(torch.float32, 1, 1, 64, 1, 8), *[torch.empty(0)] * 10)
+
+
+def test_alibi_caller_matches_oracle():
+    from eet_amd import decoder
+    from oracle import ops as O
+    assert np.allclose(decoder.alibi_slopes(40), O.alibi_slopes(40))
+    m = decoder.alibi_mask(8, 6).numpy()
+    assert np.array_equal(np.nan_to_num(m, neginf=-1), np.nan_to_num(O.alibi_mask(8, 6), neginf=-1))

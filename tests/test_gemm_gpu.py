@@ -1,0 +1,116 @@
+"""GPU parity of the fused dequant-GEMM against the fp32 oracle
+(dequantise-then-matmul), through the C ABI.  Tolerance: 1e-2 rel / 1e-3 abs."""
+import numpy as np
+import pytest
+import torch
+
+import eet_amd
+from oracle import ops as O
+
+from gpu_util import assert_close, gemm
+
+pytestmark = pytest.mark.gpu
+
+
+def make(M, K, N, seed, mode="ref128"):
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(K, N, generator=g) * 0.02).half()
+    x = torch.randn(M, K, generator=g).half()
+    u, p, s = eet_amd.quant_weights(w, torch.int8, True, mode=mode)
+    return x, u, p, s
+
+
+SMALL = [(1, 64, 16), (1, 256, 64), (3, 128, 48), (8, 1024, 176), (16, 1024, 1024), (17, 512, 48), (32, 576, 80),
+         (5, 2752, 512), (9, 4096, 112)]
+
+
+@pytest.mark.parametrize("M,K,N", SMALL)
+def test_small_shapes(gpu, M, K, N):
+    x, u, p, s = make(M, K, N, 100 + M + K + N)
+    c = gemm(x.to(gpu), p.to(gpu), s.to(gpu), M, N, K)
+    assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32), what=f"{M}x{K}x{N}")
+
+
+# BASELINE configs 1 and 2: LLaMA-7B decode linears at M in {1, 4, 8, 16, 32}
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 12288), (4096, 11008), (11008, 4096)])
+def test_llama7b_shapes(gpu, K, N):
+    x, u, p, s = make(32, K, N, K + N)
+    pd, sd = p.to(gpu), s.to(gpu)
+    ref32 = O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32)
+    for M in (1, 4, 8, 16, 32):
+        c = gemm(x[:M].contiguous().to(gpu), pd, sd, M, N, K)
+        assert_close(c.cpu().numpy(), ref32[:M], what=f"M={M} K={K} N={N}")
+
+
+def test_config1_sym127(gpu):
+    """BASELINE config 1 as worded: /127 scales, int8 in [-127, 127], M = 1."""
+    x, u, p, s = make(1, 4096, 4096, 1, mode="sym127")
+    c = gemm(x.to(gpu), p.to(gpu), s.to(gpu), 1, 4096, 4096)
+    assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32))
+
+
+def test_special_cases(gpu):
+    K = N = 128
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(16, K, generator=g).half()
+    # q = identity, scale = 1  =>  C == A exactly
+    eye = torch.eye(K, dtype=torch.int8)
+    c = gemm(x.to(gpu), eet_amd.pack_weights(eye).to(gpu), torch.ones(N).half().to(gpu), 16, N, K)
+    assert torch.equal(c.cpu(), x)
+    # a single non-zero weight (-128, the value that has no positive twin)
+    q = torch.zeros(K, N, dtype=torch.int8)
+    q[77, 5] = -128
+    c = gemm(x.to(gpu), eet_amd.pack_weights(q).to(gpu), torch.full((N,), 0.5).half().to(gpu), 16, N, K).cpu()
+    want = torch.zeros(16, N).half()
+    want[:, 5] = (x[:, 77].float() * -64).half()
+    assert torch.equal(c, want)
+    # extremes of the int8 range everywhere
+    q = torch.full((K, N), 127, dtype=torch.int8)
+    q[::2] = -128
+    s = torch.full((N,), 2.0 ** -7).half()
+    c = gemm(x.to(gpu), eet_amd.pack_weights(q).to(gpu), s.to(gpu), 16, N, K)
+    assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), q.numpy(), s.numpy(), np.float32))
+    # zero-scale column (the all-zero-column case of the quantiser: q = 127, scale = 0) gives exact zeros
+    s0 = s.clone()
+    s0[9] = 0
+    c = gemm(x.to(gpu), eet_amd.pack_weights(q).to(gpu), s0.to(gpu), 16, N, K).cpu()
+    assert (c[:, 9] == 0).all()
+
+
+def test_rows_are_independent(gpu):
+    """M = 1 equals row 0 of M = 32 bit for bit (same kernel family, same summation order per row)."""
+    x, u, p, s = make(32, 4096, 1024, 9)
+    pd, sd = p.to(gpu), s.to(gpu)
+    full = gemm(x.to(gpu), pd, sd, 32, 1024, 4096).cpu()
+    for M in (1, 7, 16):
+        part = gemm(x[:M].contiguous().to(gpu), pd, sd, M, 1024, 4096).cpu()
+        assert_close(part.numpy(), full[:M].numpy(), rtol=2e-3, atol=2e-4)
+
+
+def test_large_m_path(gpu):
+    """M > 32 (prefill sizes) takes the other kernel; same oracle."""
+    for (M, K, N) in [(33, 256, 64), (100, 512, 192), (256, 1024, 256), (2048, 512, 128)]:
+        x, u, p, s = make(M, K, N, M + K)
+        c = gemm(x.to(gpu), p.to(gpu), s.to(gpu), M, N, K)
+        assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32), what=f"M={M}")
+
+
+def test_full_size_linearity(gpu):
+    """Size-independent property at a BASELINE shape: gemm(a + b) == gemm(a) + gemm(b) within fp16 rounding,
+    and doubling the scales doubles the output exactly."""
+    K, N, M = 4096, 11008, 8
+    g = torch.Generator().manual_seed(11)
+    q = torch.randint(-128, 128, (K, N), generator=g, dtype=torch.int8)
+    p = eet_amd.pack_weights(q).to(gpu)
+    s = (torch.rand(N, generator=g) * 1e-3).half()
+    # multiples of 1/64 in [-1, 1): a + b is exact in fp16, so only the three output roundings differ
+    a = (torch.randint(-64, 64, (M, K), generator=g).float() / 64).half()
+    b = (torch.randint(-64, 64, (M, K), generator=g).float() / 64).half()
+    ab = (a.float() + b.float()).half()
+    ca, cb, cab = [gemm(t.to(gpu), p, s.to(gpu), M, N, K).float().cpu() for t in (a, b, ab)]
+    # each of the three outputs carries one fp16 rounding (2^-11 relative to its own magnitude)
+    err = (cab - (ca + cb)).abs()
+    assert (err <= 1e-3 + 1e-3 * (ca.abs() + cb.abs() + cab.abs())).all(), float(err.max())
+    c2 = gemm(a.to(gpu), p, (s * 2).to(gpu), M, N, K).float().cpu()
+    # exact, except where the smaller result is an fp16 subnormal (one subnormal step = 2^-24)
+    assert ((c2 - ca * 2).abs() <= 2.0 ** -24).all()

@@ -1,0 +1,85 @@
+"""GPU parity of the glue kernels and the prompt attention against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from eet_amd._lib import check, lib
+from oracle import ops as O
+
+from gpu_util import assert_close, stream
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("M,N", [(1, 64), (8, 4096), (3, 5120), (2, 16384), (5, 1000)])
+def test_rmsnorm(gpu, M, N):
+    g = torch.Generator().manual_seed(N)
+    x = torch.randn(M, N, generator=g).half()
+    gamma = (1 + 0.1 * torch.randn(N, generator=g)).half()
+    out = torch.empty(M, N, dtype=torch.float16, device=gpu)
+    xd, gd = x.to(gpu), gamma.to(gpu)
+    check(lib().eet_rmsnorm(xd.data_ptr(), gd.data_ptr(), out.data_ptr(), M, N, 1e-6, stream()))
+    assert_close(out.cpu().numpy(), O.rmsnorm(x.numpy(), gamma.numpy(), 1e-6), rtol=2e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("B,S,H,dh,rope,ts,t0", [(2, 5, 4, 128, 1, -1, 0), (3, 1, 4, 128, 1, 1030, 1030),
+                                                   (2, 7, 5, 64, 0, -1, 0), (1, 1, 2, 32, 1, 17, 17),
+                                                   (2, 1, 40, 128, 0, 9, 9)])
+def test_qkv_split(gpu, B, S, H, dh, rope, ts, t0):
+    g = torch.Generator().manual_seed(B + S + H)
+    cap = t0 + S + 3
+    qkv = torch.randn(B * S, 3 * H * dh, generator=g).half()
+    kc = torch.randn(B, H, cap, dh, generator=g).half()
+    vc = torch.randn(B, H, cap, dh, generator=g).half()
+    q_ref, k_ref, v_ref = O.qkv_split(qkv.numpy(), B, S, H, dh, bool(rope), ts)
+    kcn, vcn = kc.numpy().copy(), vc.numpy().copy()
+    kcn[:, :, t0:t0 + S] = k_ref
+    vcn[:, :, t0:t0 + S] = v_ref
+    qd = torch.empty(B, H, S, dh, dtype=torch.float16, device=gpu)
+    kcd, vcd = kc.to(gpu), vc.to(gpu)
+    qkvd = qkv.to(gpu)
+    check(lib().eet_qkv_split(qkvd.data_ptr(), qd.data_ptr(), kcd.data_ptr(), vcd.data_ptr(), B, S, H, dh,
+                              rope, ts, t0, cap, stream()))
+    # rotation angles reach ~1000 rad in fp32: allow a few fp16 ulps on O(1..4) values
+    assert_close(qd.cpu().numpy(), q_ref, rtol=4e-3, atol=4e-3)
+    assert_close(kcd.cpu().numpy(), kcn, rtol=4e-3, atol=4e-3)
+    assert np.array_equal(vcd.cpu().numpy(), vcn)          # v is a pure copy
+    if not rope:
+        assert np.array_equal(qd.cpu().numpy(), q_ref) and np.array_equal(kcd.cpu().numpy(), kcn)
+
+
+def test_swiglu_and_residual(gpu):
+    g = torch.Generator().manual_seed(1)
+    M, N = 8, 11008
+    gate = (torch.randn(M, N, generator=g) * 3).half()
+    up = torch.randn(M, N, generator=g).half()
+    gd, ud = gate.to(gpu), up.to(gpu)
+    check(lib().eet_swiglu(gd.data_ptr(), ud.data_ptr(), M, N, stream()))
+    assert_close(gd.cpu().numpy(), O.swiglu(gate.numpy(), up.numpy()), rtol=2e-3, atol=1e-3)
+    a = torch.randn(M, 4096, generator=g).half()
+    b = torch.randn(M, 4096, generator=g).half()
+    ad, bd = a.to(gpu), b.to(gpu)
+    check(lib().eet_residual_add(ad.data_ptr(), bd.data_ptr(), M, 4096, stream()))
+    assert np.array_equal(ad.cpu().numpy(), O.residual_add(a.numpy(), b.numpy()))
+
+
+@pytest.mark.parametrize("B,H,S,dh,use_pad,use_alibi", [(2, 3, 9, 128, False, False), (2, 2, 40, 64, True, False),
+                                                       (1, 4, 130, 128, False, True), (2, 2, 33, 32, True, True)])
+def test_prefill_attention(gpu, B, H, S, dh, use_pad, use_alibi):
+    g = torch.Generator().manual_seed(S)
+    cap = S + 5
+    q, k, v = [torch.randn(B, H, S, dh, generator=g).half() for _ in range(3)]
+    kc = torch.zeros(B, H, cap, dh).half()
+    vc = torch.zeros(B, H, cap, dh).half()
+    kc[:, :, :S], vc[:, :, :S] = k, v
+    pad = torch.tensor([0, 3][:B]) if use_pad else None
+    bias_full = O.alibi_mask(H, S) if use_alibi else None
+    want = O.prefill_attention(q.numpy(), k.numpy(), v.numpy(), pad.numpy() if use_pad else None, bias_full)
+    ctx = torch.empty(B, S, H * dh, dtype=torch.float16, device=gpu)
+    row = torch.from_numpy(O.alibi_bias(H, S)).to(gpu) if use_alibi else None
+    padd = pad.to(gpu) if use_pad else None
+    qd, kcd, vcd = q.to(gpu), kc.to(gpu), vc.to(gpu)
+    check(lib().eet_prefill_attention(qd.data_ptr(), kcd.data_ptr(), vcd.data_ptr(),
+                                      ctx.data_ptr(), row.data_ptr() if use_alibi else None,
+                                      padd.data_ptr() if use_pad else None, B, H, S, dh, cap, stream()))
+    assert_close(ctx.cpu().numpy(), want, what="prefill ctx")

@@ -1,0 +1,90 @@
+"""GPU parity of the decode attention against the fp32 oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ops as O
+
+from gpu_util import assert_close, mmha
+
+pytestmark = pytest.mark.gpu
+
+
+def case(B, H, dh, step, cap, seed, use_pad=False, use_alibi=False):
+    g = torch.Generator().manual_seed(seed)
+    kc = torch.randn(B, H, cap, dh, generator=g).half()
+    vc = torch.randn(B, H, cap, dh, generator=g).half()
+    q, k, v = [torch.randn(B, H, dh, generator=g).half() for _ in range(3)]
+    pad = torch.randint(0, max(1, step // 2), (B,), generator=g) if use_pad else None
+    alibi = torch.from_numpy(O.alibi_bias(H, step)) if use_alibi else None
+    return q, k, v, kc, vc, pad, alibi
+
+
+CASES = [
+    # B, H, dh, step, cap, pad, alibi
+    (2, 4, 128, 1, 16, False, False),
+    (2, 4, 128, 2, 16, False, False),
+    (2, 4, 128, 37, 64, True, False),
+    (3, 5, 64, 300, 512, False, True),
+    (2, 2, 32, 70, 80, True, True),
+    (1, 8, 128, 4096, 4100, False, False),      # past the reference's 4096-step limit? no: exactly at it
+    (1, 2, 128, 5000, 5000, True, False),       # beyond it
+    (8, 32, 128, 1025, 1153, False, False),     # BASELINE config 4, first decode step
+    (8, 32, 128, 1152, 1153, False, False),     # config 4, last decode step
+    (4, 40, 128, 2304, 2305, False, True),      # config 5 shape at reduced batch
+]
+
+
+@pytest.mark.parametrize("B,H,dh,step,cap,use_pad,use_alibi", CASES)
+def test_against_oracle(gpu, B, H, dh, step, cap, use_pad, use_alibi):
+    q, k, v, kc, vc, pad, alibi = case(B, H, dh, step, cap, step + B, use_pad, use_alibi)
+    kcn, vcn = kc.numpy().copy(), vc.numpy().copy()
+    want = O.decode_attention(q.numpy(), k.numpy(), v.numpy(), kcn, vcn, step,
+                              pad.numpy() if use_pad else None, alibi.numpy() if use_alibi else None)
+    kcd, vcd = kc.to(gpu), vc.to(gpu)
+    ctx = mmha(q.to(gpu), k.to(gpu), v.to(gpu), kcd, vcd, step, pad.to(gpu) if use_pad else None,
+               alibi.to(gpu) if use_alibi else None)
+    assert_close(ctx.cpu().numpy(), want, what="ctx")
+    # the new token landed in row step-1, nothing else moved
+    assert np.array_equal(kcd.cpu().numpy(), kcn) and np.array_equal(vcd.cpu().numpy(), vcn)
+
+
+def test_known_answers(gpu):
+    B, H, dh, cap = 2, 3, 128, 300
+    q, k, v, kc, vc, _, _ = case(B, H, dh, 1, cap, 5)
+    # step = 1  =>  ctx = v / (1 + 1e-6)
+    ctx = mmha(q.to(gpu), k.to(gpu), v.to(gpu), kc.to(gpu), vc.to(gpu), 1).cpu()
+    assert_close(ctx.view(B, H, dh).numpy(), v.float().numpy() / (1 + 1e-6))
+    # uniform keys  =>  ctx = mean of the values (both one block and split over several)
+    for step in (17, 290):
+        ku = k[:, :, None, :].expand(B, H, cap, dh).contiguous()
+        vcd = vc.to(gpu)
+        ctx = mmha(q.to(gpu), k.to(gpu), v.to(gpu), ku.to(gpu), vcd, step).cpu()
+        vv = vc.clone()
+        vv[:, :, step - 1] = v
+        assert_close(ctx.view(B, H, dh).numpy(), vv[:, :, :step].float().mean(2).numpy(), atol=2e-3)
+
+
+def test_fused_rows_and_no_append(gpu):
+    """q, k, v as rows of a fused [B, 3*H*dh] buffer (the Baichuan call form), and k = v = NULL
+    (cache already holds the new row)."""
+    B, H, dh, step, cap = 3, 4, 64, 50, 64
+    q, k, v, kc, vc, _, _ = case(B, H, dh, step, cap, 8)
+    fused = torch.cat([q.view(B, -1), k.view(B, -1), v.view(B, -1)], 1).contiguous().to(gpu)
+    kcn, vcn = kc.numpy().copy(), vc.numpy().copy()
+    want = O.decode_attention(q.numpy(), k.numpy(), v.numpy(), kcn, vcn, step)
+    hd = H * dh
+    kcd, vcd = kc.to(gpu), vc.to(gpu)
+    ctx = mmha(fused, fused[:, hd:], fused[:, 2 * hd:], kcd, vcd, step, stride=3 * hd)
+    assert_close(ctx.cpu().numpy(), want)
+    assert np.array_equal(kcd.cpu().numpy(), kcn)
+    ctx2 = mmha(q.to(gpu), None, None, torch.from_numpy(kcn).to(gpu), torch.from_numpy(vcn).to(gpu), step)
+    assert torch.equal(ctx2.cpu(), ctx.cpu())
+
+
+def test_everything_padded_gives_zeros(gpu):
+    B, H, dh, step, cap = 2, 2, 128, 9, 16
+    q, k, v, kc, vc, _, _ = case(B, H, dh, step, cap, 3)
+    pad = torch.tensor([step, 0])
+    ctx = mmha(q.to(gpu), k.to(gpu), v.to(gpu), kc.to(gpu), vc.to(gpu), step, pad.to(gpu)).cpu().view(B, H, dh)
+    assert not ctx[0].any() and ctx[1].any()

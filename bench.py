@@ -1,0 +1,247 @@
+#!/usr/bin/env python3
+"""Headline benchmark: int8 weight-only GEMM HBM GB/s at LLaMA-7B decode shapes,
+plus LLaMA-7B-shaped int8 decode tokens/s, on one MI355X.
+
+A "step" is one pass of the fused dequant-GEMM over every int8 linear of a
+32-layer LLaMA-7B-shaped decoder (160 launches over 6.48 GB of distinct packed
+weights, so nothing is served from the 256 MB Infinity Cache) at M = 8 rows of
+fp16 activations.  `value` is algorithmic bytes per step / time per step.
+
+Prints ONE JSON line.  Synthetic, seeded data; weights live in HBM before the
+timed region starts.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+LLAMA = dict(layers=32, hidden=4096, heads=32, d_ff=11008, vocab=32000)
+
+
+def linear_shapes(hidden, d_ff):
+    # (name, K, N) in the order a decoder layer calls them
+    return [("qkv", hidden, 3 * hidden), ("o", hidden, hidden), ("gate", hidden, d_ff), ("up", hidden, d_ff),
+            ("down", d_ff, hidden)]
+
+
+def linear_bytes(M, K, N):
+    """Algorithmic bytes of one int8 linear: each operand once."""
+    return K * N + 2 * N + 2 * M * K + 2 * M * N
+
+
+def make_weights(torch, eet, dev, layers, hidden, d_ff, seed):
+    """Per layer, per linear: (packed int8 [K, N], fp16 scales [N]) generated on
+    the GPU: W ~ N(0, 0.02^2) in fp16, quantised per output channel (reference
+    /128 rule) and permuted into the gfx950 layout."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    out = []
+    for _ in range(layers):
+        layer = {}
+        for name, K, N in linear_shapes(hidden, d_ff):
+            w = (torch.randn(K, N, generator=g, device=dev, dtype=torch.float32) * 0.02).half()
+            q, s = eet.quant_weights_torch(w, "ref128")
+            layer[name] = (eet.pack_weights_torch(q), s.half().contiguous())
+            del w, q
+        out.append(layer)
+    return out
+
+
+def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup):
+    """Returns seconds per step (one pass over all linears), measured with
+    events on the stream the kernels are launched on."""
+    st = torch.cuda.current_stream()
+    calls = []
+    for layer in weights:
+        for name, (w, s) in layer.items():
+            K, N = w.shape
+            calls.append((acts[K].data_ptr(), w.data_ptr(), s.data_ptr(), outs[N].data_ptr(), M, N, K))
+    f = lib.eet_gemm_w8a16
+    sp = st.cuda_stream
+
+    def one_pass():
+        for (a, w, s, c, m, n, k) in calls:
+            rc = f(a, w, s, c, m, n, k, None, 0, sp)
+            if rc:
+                raise RuntimeError(lib.eet_last_error().decode())
+    for _ in range(warmup):
+        one_pass()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(st)
+    for _ in range(steps):
+        one_pass()
+    e1.record(st)
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    return e0.elapsed_time(e1) * 1e-3 / steps, wall, len(calls)
+
+
+def cpu_baseline(torch, M, hidden, d_ff, seed, budget_s=12.0):
+    """The reference CPU path, timed on the host cores: torch dequantise
+    (int8 * scale -> fp32) + fp32 matmul -> fp16, for one layer's five linears
+    (the same shapes as the GPU workload; a bounded sample of it)."""
+    from oracle import cpu_path
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(seed)
+    layer = []
+    for name, K, N in linear_shapes(hidden, d_ff):
+        q = torch.randint(-128, 128, (K, N), generator=g, dtype=torch.int8)
+        s = (torch.rand(N, generator=g) * 1e-3).half()
+        x = torch.randn(M, K, generator=g).half()
+        layer.append((x, q, s))
+    nbytes = sum(linear_bytes(M, q.shape[0], q.shape[1]) for _, q, _ in layer)
+    cpu_path.dequant_matmul_layer(layer)          # warm-up
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        cpu_path.dequant_matmul_layer(layer)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or reps >= 20:
+            break
+    per_layer = el / reps
+    return {"value": round(nbytes / per_layer / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"one LLaMA-7B layer (5 int8 linears, M={M}, {nbytes / 1e6:.1f} MB algorithmic), "
+                      f"{reps} reps, torch {torch.__version__} dequant+matmul fp32, "
+                      f"{per_layer * 1e3:.1f} ms per layer"}
+
+
+def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed):
+    """LLaMA-7B-shaped int8 decoder, random init: prefill `prompt` tokens then
+    greedy-decode `gen` tokens; tokens/s = batch * gen / decode time."""
+    from eet_amd import decoder as D
+    cfg = D.DecoderConfig(num_layers=len(weights), hidden=LLAMA["hidden"], heads=LLAMA["heads"], d_ff=LLAMA["d_ff"],
+                          vocab=LLAMA["vocab"], max_batch=batch, max_prompt=prompt, max_full_seq=prompt + gen + 1)
+    g = torch.Generator(device=dev).manual_seed(seed)
+    H = cfg.hidden
+    sd = {}
+    for i, layer in enumerate(weights):
+        pre = f"layer.{i}."
+        for key, name in (("qkv", "self_attn.qkv_proj"), ("o", "self_attn.out_proj"), ("gate", "ffn.intermediate_0"),
+                          ("up", "ffn.intermediate_1"), ("down", "ffn.output")):
+            sd[pre + name + ".weight"], sd[pre + name + ".scale"] = layer[key]
+        sd[pre + "self_attn.layernorm.weight"] = (1 + 0.1 * torch.randn(H, generator=g, device=dev)).half()
+        sd[pre + "ffn.layernorm.weight"] = (1 + 0.1 * torch.randn(H, generator=g, device=dev)).half()
+    sd["embed_tokens.weight"] = (torch.randn(cfg.vocab, H, generator=g, device=dev) * 0.02).half()
+    sd["norm.weight"] = (1 + 0.1 * torch.randn(H, generator=g, device=dev)).half()
+    sd["lm_head.weight"] = (torch.randn(cfg.vocab, H, generator=g, device=dev) * 0.02).half()
+    model = D.Int8Decoder(cfg, sd, device=str(dev))
+    ids = torch.randint(0, cfg.vocab, (batch, prompt), generator=g, device=dev)
+    with torch.no_grad():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = model.logits(ids, True)
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        nxt = torch.argmax(logits[:, -1, :], dim=-1)
+        # one untimed decode step (allocations, first-touch)
+        logits = model.logits(nxt[:, None], False)
+        nxt = torch.argmax(logits[:, -1, :], dim=-1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(gen - 1):
+            logits = model.logits(nxt[:, None], False)
+            nxt = torch.argmax(logits[:, -1, :], dim=-1)
+        torch.cuda.synchronize()
+        t_dec = time.perf_counter() - t0
+    steps = gen - 1
+    ms = t_dec / steps * 1e3
+    # algorithmic HBM bytes of one token step: int8 weights + scales, KV cache read at mid length, fp16 lm_head
+    wbytes = sum(w.numel() + 2 * s.numel() for layer in weights for (w, s) in layer.values())
+    kv = len(weights) * 2 * (prompt + gen // 2) * batch * H * 2
+    step_bytes = wbytes + kv + cfg.vocab * H * 2
+    return {"tokens_per_s": round(batch * steps / t_dec, 1), "ms_per_token_step": round(ms, 3), "batch": batch,
+            "prompt": prompt, "generated": gen, "layers": len(weights), "prefill_s": round(t_prefill, 3),
+            "step_hbm_bytes": step_bytes,
+            "step_roofline_frac": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "note": "greedy decode, random-init weights, random token ids; lm_head and embedding are fp16 torch ops"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--m", type=int, default=8, help="activation rows of the headline GEMM pass")
+    ap.add_argument("--layers", type=int, default=LLAMA["layers"])
+    ap.add_argument("--gen", type=int, default=128, help="tokens to greedy-decode in the decoder leg (0 = skip)")
+    ap.add_argument("--prompt", type=int, default=1024)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the M = 1..32 sweep")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
+              "(the path has no collectives; see DESIGN.md for how it would shard).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import eet_amd as eet
+    from eet_amd._lib import lib
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP kernels have no CPU fallback.", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    L = lib()
+    hidden, d_ff = LLAMA["hidden"], LLAMA["d_ff"]
+    weights = make_weights(torch, eet, dev, args.layers, hidden, d_ff, seed=1234)
+    g = torch.Generator(device=dev).manual_seed(99)
+    acts = {K: torch.randn(32, K, generator=g, device=dev).half() for K in (hidden, d_ff)}
+    outs = {N: torch.empty(32, N, dtype=torch.float16, device=dev) for N in (3 * hidden, hidden, d_ff)}
+
+    M = args.m
+    sec, wall, launches = time_gemm_pass(torch, L, weights, acts, outs, M, args.steps, args.warmup)
+    step_bytes = sum(linear_bytes(M, w.shape[0], w.shape[1]) for layer in weights for (w, _) in layer.values())
+    gbs = step_bytes / sec / 1e9
+    per_launch_us = sec / launches * 1e6
+    result = {
+        "metric": "int8 W-only GEMM HBM GB/s (% peak) at M=1..16; LLaMA-7B int8 decode tokens/s, 1 GPU",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16 activations x int8 weights, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": f"LLaMA-7B-shaped decode linears, int8 per-channel weights: {args.layers} layers x "
+                               f"(QKV 4096x12288, O 4096x4096, gate/up 4096x11008, down 11008x4096) at M={M}",
+                   "launches_per_step": launches, "bytes_per_step": step_bytes,
+                   "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2)},
+        "roofline": {"bound": "hbm", "kernel": "w8a16_small_m_kernel", "achieved": round(gbs, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "avg_launch_us": round(per_launch_us, 3),
+                     "algorithmic_bytes_per_launch": round(step_bytes / launches), "traffic": None},
+        "host_wall_ms_per_step": round(wall * 1e3, 4),
+    }
+
+    if not args.no_sweep:
+        sweep = {}
+        for m in (1, 4, 8, 16, 32):
+            s, _, n = time_gemm_pass(torch, L, weights, acts, outs, m, max(3, args.steps // 4), 1)
+            b = sum(linear_bytes(m, w.shape[0], w.shape[1]) for layer in weights for (w, _) in layer.values())
+            sweep[f"M={m}"] = {"GB/s": round(b / s / 1e9, 1), "pct_peak": round(100 * b / s / 1e9 / HBM_PEAK_GBS, 2)}
+        per_shape = {}
+        for name, K, N in linear_shapes(hidden, d_ff):
+            sub = [{name: layer[name]} for layer in weights]
+            s, _, n = time_gemm_pass(torch, L, sub, acts, outs, M, max(3, args.steps // 4), 1)
+            b = linear_bytes(M, K, N)
+            per_shape[f"{name} K={K} N={N}"] = {"us": round(s / n * 1e6, 2), "GB/s": round(b * n / s / 1e9, 1),
+                                                "pct_peak": round(100 * b * n / s / 1e9 / HBM_PEAK_GBS, 2)}
+        result["gemm_by_m"] = sweep
+        result[f"gemm_by_shape_M{M}"] = per_shape
+
+    if args.gen > 0:
+        result["decode"] = decode_bench(torch, eet, weights, dev, args.batch, args.prompt, args.gen, seed=7)
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, M, hidden, d_ff, seed=5)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

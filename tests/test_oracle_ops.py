@@ -176,3 +176,15 @@ def test_alibi_closed_form():
     assert b[0, 0] == 0 and b[3, 10] == np.float16(np.float32(want[3]) * np.float32(10))
     m = O.alibi_mask(4, 5)
     assert np.isinf(m[0, 1, 2]) and m[2, 3, 1] == b[2 * 0 + 2, 1] * 0 + O.alibi_bias(4, 5)[2, 1]
+
+
+def test_cpu_path_matches_numpy_oracle():
+    import torch
+    from oracle import cpu_path
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((4, 256)).astype(np.float16)
+    q = rng.integers(-128, 128, (256, 48), dtype=np.int8)
+    s = (rng.random(48) * 1e-2).astype(np.float16)
+    got = cpu_path.dequant_matmul(torch.from_numpy(x), torch.from_numpy(q), torch.from_numpy(s)).numpy()
+    want = O.dequant_matmul(x, q, s)
+    assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=2e-3, atol=1e-4)

@@ -56,17 +56,23 @@ __device__ __forceinline__ half8 widen8(uint32_t x0, uint32_t x1)
     return r;
 }
 
-// One batch of U k-tiles: the raw weight tiles of NT n-tiles and the matching
-// activation operands of MT m-tiles, as they come back from memory.
-template <int NT, int MT, int U>
+// One batch of U k-tiles as it comes back from memory: the raw weight tiles of
+// NT n-tiles, and the activations of RG groups of 8 rows, loaded row-wise.
+template <int NT, int RG, int U>
 struct Batch {
     u32x4 w[U][NT];
-    u32x4 a[U][MT][2];
+    u32x4 a[U][RG];
 };
 
-template <int NT, int MT, int WAVES, int U>
-__device__ __forceinline__ void load_batch(Batch<NT, MT, U> &b, const u32x4 *const (&wbase)[NT],
-                                           const u32x4 *const (&abase)[MT], int kt)
+// Activation loads are issued so that a wavefront reads whole 128-byte lines:
+// lane l fetches the 16-byte piece l%8 of row 8*r + l/8 of the k-tile (8 rows
+// x 128 B = 1 KiB per instruction).  Letting each lane fetch its own MFMA
+// operand straight from the row-major matrix instead costs 16 half-used lines
+// per instruction and measured 1.4 us (M = 8) to 2.5 us (M = 16) on a 4 us
+// kernel.
+template <int NT, int RG, int WAVES, int U>
+__device__ __forceinline__ void load_batch(Batch<NT, RG, U> &b, const u32x4 *const (&wbase)[NT],
+                                           const u32x4 *const (&abase)[RG], int kt)
 {
     // All weight loads (HBM latency) go out first, then the activation loads
     // (L2 hits); loads return in issue order.
@@ -79,43 +85,75 @@ __device__ __forceinline__ void load_batch(Batch<NT, MT, U> &b, const u32x4 *con
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            b.a[u][mt][0] = abase[mt][(kt + u * WAVES) * 8];
-            b.a[u][mt][1] = abase[mt][(kt + u * WAVES) * 8 + 1];
-        }
+        for (int r = 0; r < RG; ++r)
+            b.a[u][r] = abase[r][(kt + u * WAVES) * 8];
     __builtin_amdgcn_sched_barrier(0);
 }
 
-template <int NT, int MT, int U>
-__device__ __forceinline__ void mma_batch(const Batch<NT, MT, U> &b, floatx4 (&acc)[NT][MT])
+// The row-wise activation pieces are turned into MFMA operands through a
+// wavefront-private LDS slab: lane (g, j) of operand half h needs piece
+// 2*g + h of row j.  Piece p of row jr is kept at slot jr*8 + (p ^ jr), which
+// makes both the 16-byte writes and the 16-byte reads bank-conflict free.
+template <int NT, int RG, int U>
+__device__ __forceinline__ void mma_batch(const Batch<NT, RG, U> &b, floatx4 (&acc)[NT][(RG + 1) / 2],
+                                          u32x4 *slab, int lane)
 {
+    constexpr int MT = (RG + 1) / 2;
+    const int g = lane >> 4, j = lane & 15;
+    const int wslot = (lane & ~7) | ((lane & 7) ^ (lane >> 3));
+    const int jr = j & 7;
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int r = 0; r < RG; ++r)
+            slab[(u * RG + r) * 64 + wslot] = b.a[u][r];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        half8 op[MT][2];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            // rows 16*mt + j; a row group that was not loaded (M <= 8 with one
+            // group) is replaced by group 0: those columns are never written
+            const int r = (2 * mt + (j >> 3) < RG) ? 2 * mt + (j >> 3) : 0;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                op[mt][h] = __builtin_bit_cast(half8, slab[(u * RG + r) * 64 + jr * 8 + ((2 * g + h) ^ jr)]);
+        }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const half8 w0 = widen8(b.w[u][t].x, b.w[u][t].y);
             const half8 w1 = widen8(b.w[u][t].z, b.w[u][t].w);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, __builtin_bit_cast(half8, b.a[u][mt][0]),
-                                                                    acc[t][mt], 0, 0, 0);
-                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, __builtin_bit_cast(half8, b.a[u][mt][1]),
-                                                                    acc[t][mt], 0, 0, 0);
+                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, op[mt][0], acc[t][mt], 0, 0, 0);
+                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, op[mt][1], acc[t][mt], 0, 0, 0);
             }
         }
+    }
 }
 
-template <int NT, int MT, int WAVES, int U>
+// NT: n-tiles per workgroup.  RG: groups of 8 activation rows (M <= 8 * RG).
+template <int NT, int RG, int WAVES, int U>
 __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
     _Float16 *__restrict__ C, int M, int N, int K)
 {
+    constexpr int MT = (RG + 1) / 2;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int g = lane >> 4, j = lane & 15;
     const int ktiles = K >> 6;
     const int ntiles = N >> 4;
     const int nt0 = blockIdx.x * NT;
+
+    // LDS: first the per-wavefront activation slabs, later (after a barrier)
+    // the partial sums of the cross-wavefront reduction.
+    constexpr int kSlabVec = U * RG * 64;                      // u32x4 per wavefront
+    constexpr int kStageBytes = WAVES * kSlabVec * 16;
+    constexpr int kRedBytes = WAVES * NT * MT * 64 * 16;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
+    u32x4 *slab = reinterpret_cast<u32x4 *>(lds) + wave * kSlabVec;
 
     floatx4 acc[NT][MT];
 #pragma unroll
@@ -131,13 +169,13 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         int nt = min(nt0 + t, ntiles - 1);
         wbase[t] = Wp + (size_t)nt * ktiles * 64 + lane;
     }
-    // Lanes whose row is past M read row M-1: column m of the product depends
-    // only on activation row m, and rows >= M are not written.
-    const u32x4 *abase[MT];
+    // Rows past M read row M-1: column m of the product depends only on
+    // activation row m, and rows >= M are not written.
+    const u32x4 *abase[RG];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        int m = min(mt * 16 + j, M - 1);
-        abase[mt] = reinterpret_cast<const u32x4 *>(A + (size_t)m * K + 16 * g);
+    for (int r = 0; r < RG; ++r) {
+        int m = min(8 * r + (lane >> 3), M - 1);
+        abase[r] = reinterpret_cast<const u32x4 *>(A + (size_t)m * K) + (lane & 7);
     }
 
     // This wavefront's k-tiles are wave, wave + WAVES, ...; they are taken in
@@ -148,27 +186,27 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     constexpr int STEP = U * WAVES;
     int kt = wave;
     {
-        Batch<NT, MT, U> b0, b1;
+        Batch<NT, RG, U> b0, b1;
         if (nbatch > 0)
-            load_batch<NT, MT, WAVES, U>(b0, wbase, abase, kt);
+            load_batch<NT, RG, WAVES, U>(b0, wbase, abase, kt);
         int i = 0;
         for (; i + 2 <= nbatch; i += 2) {
-            load_batch<NT, MT, WAVES, U>(b1, wbase, abase, kt + STEP);
-            mma_batch<NT, MT, U>(b0, acc);
+            load_batch<NT, RG, WAVES, U>(b1, wbase, abase, kt + STEP);
+            mma_batch<NT, RG, U>(b0, acc, slab, lane);
             if (i + 2 < nbatch)
-                load_batch<NT, MT, WAVES, U>(b0, wbase, abase, kt + 2 * STEP);
-            mma_batch<NT, MT, U>(b1, acc);
+                load_batch<NT, RG, WAVES, U>(b0, wbase, abase, kt + 2 * STEP);
+            mma_batch<NT, RG, U>(b1, acc, slab, lane);
             kt += 2 * STEP;
         }
         if (i < nbatch) {
-            mma_batch<NT, MT, U>(b0, acc);
+            mma_batch<NT, RG, U>(b0, acc, slab, lane);
             kt += STEP;
         }
     }
     for (; kt < ktiles; kt += WAVES) {
-        Batch<NT, MT, 1> b;
-        load_batch<NT, MT, WAVES, 1>(b, wbase, abase, kt);
-        mma_batch<NT, MT, 1>(b, acc);
+        Batch<NT, RG, 1> b;
+        load_batch<NT, RG, WAVES, 1>(b, wbase, abase, kt);
+        mma_batch<NT, RG, 1>(b, acc, slab, lane);
     }
 
     // Per-channel scales for the epilogue, requested before the barrier so
@@ -184,19 +222,20 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
 
     // Cross-wavefront reduction.  acc[t][mt][r] of lane (g, j) is the product
     // for channel 16*(nt0+t) + 4*g + r and row 16*mt + j.
-    __shared__ floatx4 red[WAVES][NT * MT][64];
+    __syncthreads();  // every wavefront is done with its activation slab
+    floatx4 *red = reinterpret_cast<floatx4 *>(lds);  // [WAVES][NT * MT][64]
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-            red[wave][t * MT + mt][lane] = acc[t][mt];
+            red[(wave * NT * MT + t * MT + mt) * 64 + lane] = acc[t][mt];
     __syncthreads();
     int idx = 0;
     for (int tile = wave; tile < NT * MT; tile += WAVES, ++idx) {
-        floatx4 s = red[0][tile][lane];
+        floatx4 s = red[tile * 64 + lane];
 #pragma unroll
         for (int w = 1; w < WAVES; ++w)
-            s += red[w][tile][lane];
+            s += red[(w * NT * MT + tile) * 64 + lane];
         const int t = tile / MT, mt = tile % MT;
         const int m = mt * 16 + j;
         if (nt0 + t < ntiles && m < M) {
@@ -215,27 +254,39 @@ struct SmallMConfig {
     int nt, waves, u;
 };
 
-template <int NT, int MT, int WAVES, int U>
+template <int NT, int RG, int WAVES, int U>
 int launch_small_m(const void *A, const void *Wp, const void *scale, void *C, int M, int N, int K, hipStream_t st)
 {
     const int ntiles = N / 16;
     dim3 grid((ntiles + NT - 1) / NT), block(WAVES * 64);
-    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, MT, WAVES, U>), grid, block, 0, st,
+    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U>), grid, block, 0, st,
                        static_cast<const _Float16 *>(A), static_cast<const u32x4 *>(Wp),
                        static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(C), M, N, K);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
 
-template <int MT>
+// LDS and register budget of an instantiation: slabs and reduction buffer within
+// 64 KiB, and the two register batches small enough not to spill.
+constexpr bool small_m_fits(int nt, int rg, int waves, int u)
+{
+    const int mt = (rg + 1) / 2;
+    const int stage = waves * u * rg * 1024, red = waves * nt * mt * 1024;
+    const int batch_vgprs = 2 * u * (nt + rg) * 4 + nt * mt * 4;
+    return stage <= 65536 && red <= 65536 && batch_vgprs <= (waves == 16 ? 96 : 200);
+}
+
+template <int RG>
 int dispatch_small_m(SmallMConfig cfg, const void *A, const void *Wp, const void *scale, void *C, int M, int N,
                      int K, hipStream_t st)
 {
-#define EET_CASE(NT_, W_, U_)                                 \
-    if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_)      \
-        return launch_small_m<NT_, MT, W_, U_>(A, Wp, scale, C, M, N, K, st);
-    EET_CASE(1, 4, 4) EET_CASE(1, 8, 4) EET_CASE(1, 16, 4) EET_CASE(1, 8, 2) EET_CASE(1, 16, 2)
-    EET_CASE(2, 4, 2) EET_CASE(2, 8, 2) EET_CASE(2, 16, 2) EET_CASE(2, 8, 4) EET_CASE(2, 16, 1)
+#define EET_CASE(NT_, W_, U_)                                                            \
+    if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_) {                               \
+        if constexpr (small_m_fits(NT_, RG, W_, U_))                                     \
+            return launch_small_m<NT_, RG, W_, U_>(A, Wp, scale, C, M, N, K, st);        \
+    }
+    EET_CASE(1, 4, 4) EET_CASE(1, 8, 4) EET_CASE(1, 16, 4) EET_CASE(1, 8, 2) EET_CASE(1, 16, 2) EET_CASE(1, 16, 1)
+    EET_CASE(2, 4, 2) EET_CASE(2, 8, 2) EET_CASE(2, 16, 2) EET_CASE(2, 8, 4) EET_CASE(2, 16, 1) EET_CASE(2, 8, 1)
     EET_CASE(3, 8, 2) EET_CASE(3, 16, 2) EET_CASE(3, 16, 1) EET_CASE(3, 8, 1)
     EET_CASE(4, 4, 2) EET_CASE(4, 8, 2) EET_CASE(4, 8, 1) EET_CASE(4, 16, 1)
 #undef EET_CASE
@@ -253,22 +304,21 @@ SmallMConfig pick_small_m(int M, int N, int K)
         if (sscanf(env, "%d,%d,%d", &c.nt, &c.waves, &c.u) == 3)
             return c;
     }
-    // Measured on MI355X (LLaMA-7B shapes, M = 1..32): three n-tiles per
-    // workgroup reuse each activation operand three times and win whenever
-    // that still leaves >= ~200 workgroups; otherwise one n-tile per
-    // workgroup, with 16 wavefronts once K is long enough to feed them.
+    // Measured on MI355X (LLaMA-7B shapes, M = 1..32).  Every workgroup reads
+    // all M x K activations once, so with enough n-tiles three of them per
+    // workgroup (activation operand reused three times) win as soon as M > 4;
+    // with few n-tiles one per workgroup is needed to occupy the 256 CUs, and
+    // 16 wavefronts keep enough loads in flight.
     const int ntiles = N / 16;
     SmallMConfig c;
     if (ntiles >= 600) {
-        c = SmallMConfig{3, 8, 1};
+        c = (M <= 4) ? SmallMConfig{1, 8, 2} : SmallMConfig{3, 8, 1};
     } else if (ntiles >= 400) {
         c = SmallMConfig{2, 8, 2};
-    } else if (K >= 8192 && M <= 16) {
-        c = SmallMConfig{1, 16, 2};
     } else {
-        c = SmallMConfig{1, 8, 2};
+        c = (M > 16) ? SmallMConfig{1, 16, 1} : SmallMConfig{1, 16, 2};
     }
-    (void)M;
+    (void)K;
     return c;
 }
 
@@ -295,9 +345,11 @@ extern "C" int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *sc
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (M <= 32) {
         SmallMConfig cfg = pick_small_m(M, N, K);
-        if (M <= 16)
+        if (M <= 8)
             return dispatch_small_m<1>(cfg, A, Wpacked, scale, C, M, N, K, st);
-        return dispatch_small_m<2>(cfg, A, Wpacked, scale, C, M, N, K, st);
+        if (M <= 16)
+            return dispatch_small_m<2>(cfg, A, Wpacked, scale, C, M, N, K, st);
+        return dispatch_small_m<4>(cfg, A, Wpacked, scale, C, M, N, K, st);
     }
     return eet_gemm_w8a16_large_m(A, Wpacked, scale, C, M, N, K, st);
 }
@@ -312,8 +364,9 @@ int eet_gemm_w8a16_large_m(const void *A, const void *Wp, const void *scale, voi
         const int mm = (M - m0 < 32) ? M - m0 : 32;
         const _Float16 *a = static_cast<const _Float16 *>(A) + (size_t)m0 * K;
         _Float16 *c = static_cast<_Float16 *>(C) + (size_t)m0 * N;
-        int rc = (mm <= 16) ? dispatch_small_m<1>(cfg, a, Wp, scale, c, mm, N, K, st)
-                            : dispatch_small_m<2>(cfg, a, Wp, scale, c, mm, N, K, st);
+        int rc = (mm <= 8)    ? dispatch_small_m<1>(cfg, a, Wp, scale, c, mm, N, K, st)
+                 : (mm <= 16) ? dispatch_small_m<2>(cfg, a, Wp, scale, c, mm, N, K, st)
+                              : dispatch_small_m<4>(cfg, a, Wp, scale, c, mm, N, K, st);
         if (rc)
             return rc;
     }

@@ -26,9 +26,9 @@ FLAGS = [
 def build(verbose=True):
     objs = []
     procs = []
-    os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    os.makedirs(os.path.join(HERE, "_obj"), exist_ok=True)
     for src in SOURCES:
-        obj = os.path.join(HERE, "build", src + ".o")
+        obj = os.path.join(HERE, "_obj", src + ".o")
         cmd = [HIPCC] + [f for f in FLAGS if f != "-shared"] + ["-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)

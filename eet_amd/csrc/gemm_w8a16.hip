@@ -322,10 +322,172 @@ SmallMConfig pick_small_m(int M, int N, int K)
     return c;
 }
 
+// ---------------------------------------------------------------------------
+// Large-M kernel (M > 32, prefill; fp16-MFMA bound).
+//
+// Block tile 128 (M) x 256 (N) x 64 (K), 4 wavefronts side by side along N,
+// each 128 x 64 = 8 m-tiles x 4 n-tiles of v_mfma_f32_16x16x32_f16 (128 fp32
+// accumulator registers).  Weights: every wavefront reads its own four packed
+// tiles straight from global memory into registers -- the packed layout is
+// already the MFMA operand layout, so they never touch LDS -- and widens them
+// once per k-tile.  Activations: the block's 128 x 64 slab is loaded row-wise
+// (whole 128-byte lines), written to LDS in operand order with an XOR swizzle
+// (conflict-free 16-byte writes and reads) and read by all four wavefronts.
+// Both streams are prefetched one k-tile ahead; one barrier per k-tile.
+// Workgroups are numbered so that the ones sharing a weight column block run
+// on the same XCD (workgroup i lands on XCD i % 8) and hit its L2.
+// ---------------------------------------------------------------------------
+constexpr int kLmBM = 128, kLmBN = 256, kLmTM = kLmBM / 16, kLmTN = 4;
+
+__global__ __launch_bounds__(256) void w8a16_large_m_kernel(const _Float16 *__restrict__ A,
+                                                            const u32x4 *__restrict__ Wp,
+                                                            const _Float16 *__restrict__ scale,
+                                                            _Float16 *__restrict__ C, int M, int N, int K,
+                                                            int m_blocks, int n_blocks)
+{
+    __shared__ u32x4 lds[2][kLmTM * 2 * 64];  // [buffer][(mt*2+h)*64 + slot], 16 KiB each
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = lane >> 4, j = lane & 15;
+    const int ktiles = K >> 6, ntiles = N >> 4;
+
+    // XCD-aware tile order: consecutive workgroups of one XCD walk down the
+    // m-blocks of the same n-block.
+    const int total = m_blocks * n_blocks;
+    const int per_xcd = (total + 7) / 8;
+    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (tile >= total)
+        return;
+    const int n_blk = tile / m_blocks, m_blk = tile % m_blocks;
+    const int m0 = m_blk * kLmBM;
+    const int nt0 = n_blk * (kLmBN / 16) + wave * kLmTN;
+
+    const u32x4 *wbase[kLmTN];
+#pragma unroll
+    for (int t = 0; t < kLmTN; ++t)
+        wbase[t] = Wp + (size_t)min(nt0 + t, ntiles - 1) * ktiles * 64 + lane;
+
+    // activation pieces: 128 rows x 8 pieces of 16 bytes = 1024, four per thread
+    const u32x4 *asrc[4];
+    int adst[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int q = tid + 256 * i, row = q >> 3, p = q & 7;
+        asrc[i] = reinterpret_cast<const u32x4 *>(A + (size_t)min(m0 + row, M - 1) * K) + p;
+        adst[i] = ((row >> 4) * 2 + (p & 1)) * 64 + (p >> 1) * 16 + ((row & 15) ^ p);
+    }
+
+    floatx4 acc[kLmTN][kLmTM];
+#pragma unroll
+    for (int t = 0; t < kLmTN; ++t)
+#pragma unroll
+        for (int mt = 0; mt < kLmTM; ++mt)
+            acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    u32x4 wcur[kLmTN], wnext[kLmTN], areg[4];
+#pragma unroll
+    for (int t = 0; t < kLmTN; ++t)
+        wcur[t] = wbase[t][0];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        areg[i] = asrc[i][0];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        lds[0][adst[i]] = areg[i];
+    __syncthreads();
+
+    const int rslot0 = g * 16 + (j ^ (2 * g)), rslot1 = g * 16 + (j ^ (2 * g + 1));
+    for (int kt = 0; kt < ktiles; ++kt) {
+        const bool more = kt + 1 < ktiles;
+        if (more) {
+#pragma unroll
+            for (int t = 0; t < kLmTN; ++t)
+                wnext[t] = wbase[t][(size_t)(kt + 1) * 64];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                areg[i] = asrc[i][(kt + 1) * 8];
+        }
+        half8 w0[kLmTN], w1[kLmTN];
+#pragma unroll
+        for (int t = 0; t < kLmTN; ++t) {
+            w0[t] = widen8(wcur[t].x, wcur[t].y);
+            w1[t] = widen8(wcur[t].z, wcur[t].w);
+        }
+        const u32x4 *buf = lds[kt & 1];
+#pragma unroll
+        for (int mt = 0; mt < kLmTM; ++mt) {
+            const half8 a0 = __builtin_bit_cast(half8, buf[(mt * 2) * 64 + rslot0]);
+            const half8 a1 = __builtin_bit_cast(half8, buf[(mt * 2 + 1) * 64 + rslot1]);
+#pragma unroll
+            for (int t = 0; t < kLmTN; ++t) {
+                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0[t], a0, acc[t][mt], 0, 0, 0);
+                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1[t], a1, acc[t][mt], 0, 0, 0);
+            }
+        }
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                lds[(kt + 1) & 1][adst[i]] = areg[i];
+#pragma unroll
+            for (int t = 0; t < kLmTN; ++t)
+                wcur[t] = wnext[t];
+        }
+        __syncthreads();
+    }
+
+    // acc[t][mt][r] of lane (g, j): row m0 + 16*mt + j, channel 16*(nt0+t) + 4*g + r
+#pragma unroll
+    for (int t = 0; t < kLmTN; ++t) {
+        if (nt0 + t >= ntiles)
+            continue;
+        const int n = (nt0 + t) * 16 + 4 * g;
+        const half4 sc = *reinterpret_cast<const half4 *>(scale + n);
+        const float s0 = (float)sc.x, s1 = (float)sc.y, s2 = (float)sc.z, s3 = (float)sc.w;
+#pragma unroll
+        for (int mt = 0; mt < kLmTM; ++mt) {
+            const int m = m0 + 16 * mt + j;
+            if (m < M) {
+                half4 o;
+                o.x = (_Float16)(acc[t][mt].x * s0);
+                o.y = (_Float16)(acc[t][mt].y * s1);
+                o.z = (_Float16)(acc[t][mt].z * s2);
+                o.w = (_Float16)(acc[t][mt].w * s3);
+                *reinterpret_cast<half4 *>(C + (size_t)m * N + n) = o;
+            }
+        }
+    }
+}
+
 }  // namespace
 
-int eet_gemm_w8a16_large_m(const void *A, const void *Wp, const void *scale, void *C, int M, int N, int K,
-                           hipStream_t st);
+static int eet_gemm_w8a16_large_m(const void *A, const void *Wp, const void *scale, void *C, int M, int N, int K,
+                                  hipStream_t st)
+{
+    if (M <= 128) {
+        // Too few 128 x 256 tiles to occupy the chip: run the small-M kernel over
+        // 32-row slabs instead (the weights are re-read per slab, from L2 / Infinity Cache).
+        SmallMConfig cfg = pick_small_m(32, N, K);
+        for (int m0 = 0; m0 < M; m0 += 32) {
+            const int mm = (M - m0 < 32) ? M - m0 : 32;
+            const _Float16 *a = static_cast<const _Float16 *>(A) + (size_t)m0 * K;
+            _Float16 *c = static_cast<_Float16 *>(C) + (size_t)m0 * N;
+            int rc = (mm <= 8)    ? dispatch_small_m<1>(pick_small_m(mm, N, K), a, Wp, scale, c, mm, N, K, st)
+                     : (mm <= 16) ? dispatch_small_m<2>(pick_small_m(mm, N, K), a, Wp, scale, c, mm, N, K, st)
+                                  : dispatch_small_m<4>(cfg, a, Wp, scale, c, mm, N, K, st);
+            if (rc)
+                return rc;
+        }
+        return EET_OK;
+    }
+    const int m_blocks = (M + kLmBM - 1) / kLmBM, n_blocks = (N + kLmBN - 1) / kLmBN;
+    const int total = m_blocks * n_blocks;
+    const int grid = ((total + 7) / 8) * 8;
+    hipLaunchKernelGGL(w8a16_large_m_kernel, dim3(grid), dim3(256), 0, st, static_cast<const _Float16 *>(A),
+                       static_cast<const u32x4 *>(Wp), static_cast<const _Float16 *>(scale),
+                       static_cast<_Float16 *>(C), M, N, K, m_blocks, n_blocks);
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
 
 extern "C" int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *scale, void *C, int M, int N, int K,
                               void *workspace, size_t workspace_bytes, void *stream)
@@ -352,23 +514,4 @@ extern "C" int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *sc
         return dispatch_small_m<4>(cfg, A, Wpacked, scale, C, M, N, K, st);
     }
     return eet_gemm_w8a16_large_m(A, Wpacked, scale, C, M, N, K, st);
-}
-
-// Interim large-M path: the small-M kernel over 32-row slabs (re-reads the
-// weights once per slab).
-int eet_gemm_w8a16_large_m(const void *A, const void *Wp, const void *scale, void *C, int M, int N, int K,
-                           hipStream_t st)
-{
-    SmallMConfig cfg = pick_small_m(32, N, K);
-    for (int m0 = 0; m0 < M; m0 += 32) {
-        const int mm = (M - m0 < 32) ? M - m0 : 32;
-        const _Float16 *a = static_cast<const _Float16 *>(A) + (size_t)m0 * K;
-        _Float16 *c = static_cast<_Float16 *>(C) + (size_t)m0 * N;
-        int rc = (mm <= 8)    ? dispatch_small_m<1>(cfg, a, Wp, scale, c, mm, N, K, st)
-                 : (mm <= 16) ? dispatch_small_m<2>(cfg, a, Wp, scale, c, mm, N, K, st)
-                              : dispatch_small_m<4>(cfg, a, Wp, scale, c, mm, N, K, st);
-        if (rc)
-            return rc;
-    }
-    return EET_OK;
 }

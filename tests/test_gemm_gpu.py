@@ -89,7 +89,8 @@ def test_rows_are_independent(gpu):
 
 def test_large_m_path(gpu):
     """M > 32 (prefill sizes) takes the other kernel; same oracle."""
-    for (M, K, N) in [(33, 256, 64), (100, 512, 192), (256, 1024, 256), (2048, 512, 128)]:
+    for (M, K, N) in [(33, 256, 64), (100, 512, 192), (129, 256, 48), (256, 1024, 256), (300, 576, 272),
+                      (2048, 512, 128), (2048, 5120, 512)]:
         x, u, p, s = make(M, K, N, M + K)
         c = gemm(x.to(gpu), p.to(gpu), s.to(gpu), M, N, K)
         assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32), what=f"M={M}")

@@ -56,6 +56,10 @@ __device__ __forceinline__ half8 widen8(uint32_t x0, uint32_t x1)
     return r;
 }
 
+// Epilogues: plain; + residual[M][N] (fp16 add); SwiGLU over (gate, up) n-tile
+// pairs of an interleaved weight, output [M][N/2].
+constexpr int kEpiNone = 0, kEpiResidual = 1, kEpiSwiglu = 2;
+
 // One batch of U k-tiles as it comes back from memory: the raw weight tiles of
 // NT n-tiles, and the activations of RG groups of 8 rows, loaded row-wise.
 template <int NT, int RG, int U>
@@ -137,7 +141,7 @@ __device__ __forceinline__ void mma_batch(const Batch<NT, RG, U> &b, floatx4 (&a
 template <int NT, int RG, int WAVES, int U>
 __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
-    _Float16 *__restrict__ C, int M, int N, int K)
+    _Float16 *__restrict__ C, int M, int N, int K, const _Float16 *__restrict__ residual, int epi)
 {
     constexpr int MT = (RG + 1) / 2;
     const int lane = threadIdx.x & 63;
@@ -209,14 +213,26 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         mma_batch<NT, RG, 1>(b, acc, slab, lane);
     }
 
-    // Per-channel scales for the epilogue, requested before the barrier so
-    // their latency overlaps the reduction.
-    half4 sc[(NT * MT + WAVES - 1) / WAVES];
+    // Epilogue operands (per-channel scales, residual rows) are requested before
+    // the barrier so their latency overlaps the reduction.  An output unit is
+    // one (n-tile, m-tile) product, or for the SwiGLU epilogue the pair of
+    // adjacent n-tiles (gate, up) of one m-tile.
+    constexpr int kMaxUnits = (NT * MT + WAVES - 1) / WAVES;
+    const int units = (epi == kEpiSwiglu) ? (NT / 2) * MT : NT * MT;
+    half4 sc0[kMaxUnits], sc1[kMaxUnits], res[kMaxUnits];
     {
         int idx = 0;
-        for (int tile = wave; tile < NT * MT; tile += WAVES, ++idx) {
-            const int nt = min(nt0 + tile / MT, ntiles - 1);
-            sc[idx] = *reinterpret_cast<const half4 *>(scale + nt * 16 + 4 * g);
+        for (int unit = wave; unit < units; unit += WAVES, ++idx) {
+            const int mt = unit % MT;
+            const int t = (epi == kEpiSwiglu) ? 2 * (unit / MT) : unit / MT;
+            const int nt = min(nt0 + t, ntiles - 1);
+            sc0[idx] = *reinterpret_cast<const half4 *>(scale + nt * 16 + 4 * g);
+            if (epi == kEpiSwiglu)
+                sc1[idx] = *reinterpret_cast<const half4 *>(scale + min(nt + 1, ntiles - 1) * 16 + 4 * g);
+            if (epi == kEpiResidual) {
+                const int m = min(mt * 16 + j, M - 1);
+                res[idx] = *reinterpret_cast<const half4 *>(residual + (size_t)m * N + nt * 16 + 4 * g);
+            }
         }
     }
 
@@ -230,22 +246,45 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         for (int mt = 0; mt < MT; ++mt)
             red[(wave * NT * MT + t * MT + mt) * 64 + lane] = acc[t][mt];
     __syncthreads();
-    int idx = 0;
-    for (int tile = wave; tile < NT * MT; tile += WAVES, ++idx) {
+    auto tile_sum = [&](int tile) {
         floatx4 s = red[tile * 64 + lane];
 #pragma unroll
         for (int w = 1; w < WAVES; ++w)
             s += red[(w * NT * MT + tile) * 64 + lane];
-        const int t = tile / MT, mt = tile % MT;
+        return s;
+    };
+    int idx = 0;
+    for (int unit = wave; unit < units; unit += WAVES, ++idx) {
+        const int mt = unit % MT;
         const int m = mt * 16 + j;
-        if (nt0 + t < ntiles && m < M) {
-            const int n = (nt0 + t) * 16 + 4 * g;
-            half4 o;
-            o.x = (_Float16)(s.x * (float)sc[idx].x);
-            o.y = (_Float16)(s.y * (float)sc[idx].y);
-            o.z = (_Float16)(s.z * (float)sc[idx].z);
-            o.w = (_Float16)(s.w * (float)sc[idx].w);
-            *reinterpret_cast<half4 *>(C + (size_t)m * N + n) = o;
+        if (epi == kEpiSwiglu) {
+            const int t = 2 * (unit / MT);
+            const floatx4 sg = tile_sum(t * MT + mt), su = tile_sum((t + 1) * MT + mt);
+            if (nt0 + t + 1 < ntiles && m < M) {
+                // gate and up are rounded to fp16 first, as the separate GEMMs would leave them
+                half4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float gate = (float)(_Float16)(sg[r] * (float)sc0[idx][r]);
+                    const float up = (float)(_Float16)(su[r] * (float)sc1[idx][r]);
+                    o[r] = (_Float16)(up * gate / (1.0f + __expf(-gate)));
+                }
+                const int n = ((nt0 + t) / 2) * 16 + 4 * g;
+                *reinterpret_cast<half4 *>(C + (size_t)m * (N / 2) + n) = o;
+            }
+        } else {
+            const int t = unit / MT;
+            const floatx4 s = tile_sum(unit);
+            if (nt0 + t < ntiles && m < M) {
+                const int n = (nt0 + t) * 16 + 4 * g;
+                half4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    o[r] = (_Float16)(s[r] * (float)sc0[idx][r]);
+                if (epi == kEpiResidual)
+                    o = o + res[idx];  // fp16 add of the rounded product, like the separate kernel
+                *reinterpret_cast<half4 *>(C + (size_t)m * N + n) = o;
+            }
         }
     }
 }
@@ -254,14 +293,24 @@ struct SmallMConfig {
     int nt, waves, u;
 };
 
+struct GemmArgs {
+    const _Float16 *A;
+    const u32x4 *Wp;
+    const _Float16 *scale;
+    _Float16 *C;
+    int M, N, K;
+    const _Float16 *residual;
+    int epi;
+    hipStream_t st;
+};
+
 template <int NT, int RG, int WAVES, int U>
-int launch_small_m(const void *A, const void *Wp, const void *scale, void *C, int M, int N, int K, hipStream_t st)
+int launch_small_m(const GemmArgs &a)
 {
-    const int ntiles = N / 16;
+    const int ntiles = a.N / 16;
     dim3 grid((ntiles + NT - 1) / NT), block(WAVES * 64);
-    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U>), grid, block, 0, st,
-                       static_cast<const _Float16 *>(A), static_cast<const u32x4 *>(Wp),
-                       static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(C), M, N, K);
+    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U>), grid, block, 0, a.st, a.A, a.Wp, a.scale, a.C, a.M,
+                       a.N, a.K, a.residual, a.epi);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
@@ -277,49 +326,55 @@ constexpr bool small_m_fits(int nt, int rg, int waves, int u)
 }
 
 template <int RG>
-int dispatch_small_m(SmallMConfig cfg, const void *A, const void *Wp, const void *scale, void *C, int M, int N,
-                     int K, hipStream_t st)
+int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a)
 {
-#define EET_CASE(NT_, W_, U_)                                                            \
-    if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_) {                               \
-        if constexpr (small_m_fits(NT_, RG, W_, U_))                                     \
-            return launch_small_m<NT_, RG, W_, U_>(A, Wp, scale, C, M, N, K, st);        \
+#define EET_CASE(NT_, W_, U_)                                      \
+    if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_) {         \
+        if constexpr (small_m_fits(NT_, RG, W_, U_))               \
+            return launch_small_m<NT_, RG, W_, U_>(a);             \
     }
     EET_CASE(1, 4, 4) EET_CASE(1, 8, 4) EET_CASE(1, 16, 4) EET_CASE(1, 8, 2) EET_CASE(1, 16, 2) EET_CASE(1, 16, 1)
     EET_CASE(2, 4, 2) EET_CASE(2, 8, 2) EET_CASE(2, 16, 2) EET_CASE(2, 8, 4) EET_CASE(2, 16, 1) EET_CASE(2, 8, 1)
     EET_CASE(3, 8, 2) EET_CASE(3, 16, 2) EET_CASE(3, 16, 1) EET_CASE(3, 8, 1)
     EET_CASE(4, 4, 2) EET_CASE(4, 8, 2) EET_CASE(4, 8, 1) EET_CASE(4, 16, 1)
 #undef EET_CASE
-    return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no small-M kernel for nt=%d waves=%d u=%d", cfg.nt,
-                     cfg.waves, cfg.u);
+    return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no small-M kernel for nt=%d waves=%d u=%d (M=%d)",
+                     cfg.nt, cfg.waves, cfg.u, a.M);
 }
 
-// Shape -> launch shape.  The chip has 256 CUs; aim for a few workgroups per
-// CU while keeping every wavefront at least a few k-tiles deep.
-SmallMConfig pick_small_m(int M, int N, int K)
+// Shape -> launch shape.  Measured on MI355X (LLaMA-7B shapes, M = 1..32).
+// Every workgroup reads all M x K activations once, so with enough n-tiles
+// three of them per workgroup (activation operand reused three times) win as
+// soon as M > 4; with few n-tiles one per workgroup is needed to occupy the
+// 256 CUs, and 16 wavefronts keep enough loads in flight.  The SwiGLU epilogue
+// needs an even number of n-tiles per workgroup (gate / up pairs).
+SmallMConfig pick_small_m(int M, int N, int K, int epi)
 {
     const char *env = std::getenv("EET_GEMM_SMALL_M_CONFIG");  // "nt,waves,u": tuning override
     if (env) {
         SmallMConfig c{1, 8, 4};
-        if (sscanf(env, "%d,%d,%d", &c.nt, &c.waves, &c.u) == 3)
+        if (sscanf(env, "%d,%d,%d", &c.nt, &c.waves, &c.u) == 3 && (epi != kEpiSwiglu || c.nt % 2 == 0))
             return c;
     }
-    // Measured on MI355X (LLaMA-7B shapes, M = 1..32).  Every workgroup reads
-    // all M x K activations once, so with enough n-tiles three of them per
-    // workgroup (activation operand reused three times) win as soon as M > 4;
-    // with few n-tiles one per workgroup is needed to occupy the 256 CUs, and
-    // 16 wavefronts keep enough loads in flight.
     const int ntiles = N / 16;
-    SmallMConfig c;
-    if (ntiles >= 600) {
-        c = (M <= 4) ? SmallMConfig{1, 8, 2} : SmallMConfig{3, 8, 1};
-    } else if (ntiles >= 400) {
-        c = SmallMConfig{2, 8, 2};
-    } else {
-        c = (M > 16) ? SmallMConfig{1, 16, 1} : SmallMConfig{1, 16, 2};
-    }
     (void)K;
-    return c;
+    if (epi == kEpiSwiglu)
+        return (M > 16) ? SmallMConfig{2, 8, 1} : SmallMConfig{2, 8, 2};
+    if (ntiles >= 600)
+        return (M <= 4) ? SmallMConfig{1, 8, 2} : SmallMConfig{3, 8, 1};
+    if (ntiles >= 400)
+        return (M > 16) ? SmallMConfig{2, 8, 1} : SmallMConfig{2, 8, 2};
+    return (M > 16) ? SmallMConfig{1, 16, 1} : SmallMConfig{1, 16, 2};
+}
+
+int run_small_m(const GemmArgs &a)
+{
+    const SmallMConfig cfg = pick_small_m(a.M, a.N, a.K, a.epi);
+    if (a.M <= 8)
+        return dispatch_small_m<1>(cfg, a);
+    if (a.M <= 16)
+        return dispatch_small_m<2>(cfg, a);
+    return dispatch_small_m<4>(cfg, a);
 }
 
 // ---------------------------------------------------------------------------
@@ -343,7 +398,8 @@ __global__ __launch_bounds__(256) void w8a16_large_m_kernel(const _Float16 *__re
                                                             const u32x4 *__restrict__ Wp,
                                                             const _Float16 *__restrict__ scale,
                                                             _Float16 *__restrict__ C, int M, int N, int K,
-                                                            int m_blocks, int n_blocks)
+                                                            int m_blocks, int n_blocks,
+                                                            const _Float16 *__restrict__ residual, int epi)
 {
     __shared__ u32x4 lds[2][kLmTM * 2 * 64];  // [buffer][(mt*2+h)*64 + slot], 16 KiB each
 
@@ -436,22 +492,47 @@ __global__ __launch_bounds__(256) void w8a16_large_m_kernel(const _Float16 *__re
     }
 
     // acc[t][mt][r] of lane (g, j): row m0 + 16*mt + j, channel 16*(nt0+t) + 4*g + r
+    if (epi == kEpiSwiglu) {
+#pragma unroll
+        for (int t = 0; t < kLmTN; t += 2) {
+            if (nt0 + t + 1 >= ntiles)
+                continue;
+            const half4 sg = *reinterpret_cast<const half4 *>(scale + (nt0 + t) * 16 + 4 * g);
+            const half4 su = *reinterpret_cast<const half4 *>(scale + (nt0 + t + 1) * 16 + 4 * g);
+            const int n = ((nt0 + t) / 2) * 16 + 4 * g;
+#pragma unroll
+            for (int mt = 0; mt < kLmTM; ++mt) {
+                const int m = m0 + 16 * mt + j;
+                if (m < M) {
+                    half4 o;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float gate = (float)(_Float16)(acc[t][mt][r] * (float)sg[r]);
+                        const float up = (float)(_Float16)(acc[t + 1][mt][r] * (float)su[r]);
+                        o[r] = (_Float16)(up * gate / (1.0f + __expf(-gate)));
+                    }
+                    *reinterpret_cast<half4 *>(C + (size_t)m * (N / 2) + n) = o;
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int t = 0; t < kLmTN; ++t) {
         if (nt0 + t >= ntiles)
             continue;
         const int n = (nt0 + t) * 16 + 4 * g;
         const half4 sc = *reinterpret_cast<const half4 *>(scale + n);
-        const float s0 = (float)sc.x, s1 = (float)sc.y, s2 = (float)sc.z, s3 = (float)sc.w;
 #pragma unroll
         for (int mt = 0; mt < kLmTM; ++mt) {
             const int m = m0 + 16 * mt + j;
             if (m < M) {
                 half4 o;
-                o.x = (_Float16)(acc[t][mt].x * s0);
-                o.y = (_Float16)(acc[t][mt].y * s1);
-                o.z = (_Float16)(acc[t][mt].z * s2);
-                o.w = (_Float16)(acc[t][mt].w * s3);
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    o[r] = (_Float16)(acc[t][mt][r] * (float)sc[r]);
+                if (epi == kEpiResidual)
+                    o = o + *reinterpret_cast<const half4 *>(residual + (size_t)m * N + n);
                 *reinterpret_cast<half4 *>(C + (size_t)m * N + n) = o;
             }
         }
@@ -460,32 +541,45 @@ __global__ __launch_bounds__(256) void w8a16_large_m_kernel(const _Float16 *__re
 
 }  // namespace
 
-static int eet_gemm_w8a16_large_m(const void *A, const void *Wp, const void *scale, void *C, int M, int N, int K,
-                                  hipStream_t st)
+static int run_gemm(const GemmArgs &a)
 {
-    if (M <= 128) {
+    if (a.M <= 32)
+        return run_small_m(a);
+    if (a.M <= 128) {
         // Too few 128 x 256 tiles to occupy the chip: run the small-M kernel over
         // 32-row slabs instead (the weights are re-read per slab, from L2 / Infinity Cache).
-        SmallMConfig cfg = pick_small_m(32, N, K);
-        for (int m0 = 0; m0 < M; m0 += 32) {
-            const int mm = (M - m0 < 32) ? M - m0 : 32;
-            const _Float16 *a = static_cast<const _Float16 *>(A) + (size_t)m0 * K;
-            _Float16 *c = static_cast<_Float16 *>(C) + (size_t)m0 * N;
-            int rc = (mm <= 8)    ? dispatch_small_m<1>(pick_small_m(mm, N, K), a, Wp, scale, c, mm, N, K, st)
-                     : (mm <= 16) ? dispatch_small_m<2>(pick_small_m(mm, N, K), a, Wp, scale, c, mm, N, K, st)
-                                  : dispatch_small_m<4>(cfg, a, Wp, scale, c, mm, N, K, st);
-            if (rc)
+        const int n_out = (a.epi == kEpiSwiglu) ? a.N / 2 : a.N;
+        for (int m0 = 0; m0 < a.M; m0 += 32) {
+            GemmArgs s = a;
+            s.M = (a.M - m0 < 32) ? a.M - m0 : 32;
+            s.A = a.A + (size_t)m0 * a.K;
+            s.C = a.C + (size_t)m0 * n_out;
+            if (a.residual)
+                s.residual = a.residual + (size_t)m0 * a.N;
+            if (int rc = run_small_m(s))
                 return rc;
         }
         return EET_OK;
     }
-    const int m_blocks = (M + kLmBM - 1) / kLmBM, n_blocks = (N + kLmBN - 1) / kLmBN;
+    const int m_blocks = (a.M + kLmBM - 1) / kLmBM, n_blocks = (a.N + kLmBN - 1) / kLmBN;
     const int total = m_blocks * n_blocks;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL(w8a16_large_m_kernel, dim3(grid), dim3(256), 0, st, static_cast<const _Float16 *>(A),
-                       static_cast<const u32x4 *>(Wp), static_cast<const _Float16 *>(scale),
-                       static_cast<_Float16 *>(C), M, N, K, m_blocks, n_blocks);
+    hipLaunchKernelGGL(w8a16_large_m_kernel, dim3(grid), dim3(256), 0, a.st, a.A, a.Wp, a.scale, a.C, a.M, a.N, a.K,
+                       m_blocks, n_blocks, a.residual, a.epi);
     EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
+static int check_gemm_args(const char *fn, const void *A, const void *W, const void *scale, const void *C, int M,
+                           int N, int K)
+{
+    EET_REQUIRE(A && W && scale && C, EET_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+    EET_REQUIRE(M >= 0 && N > 0 && K > 0, EET_ERR_INVALID_ARGUMENT, "%s: bad sizes M=%d N=%d K=%d", fn, M, N, K);
+    EET_REQUIRE(K % 64 == 0 && N % 16 == 0, EET_ERR_UNSUPPORTED_SHAPE,
+                "%s: need K %% 64 == 0 and N %% 16 == 0, got K=%d N=%d", fn, K, N);
+    EET_REQUIRE((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W)) % 16 == 0 &&
+                    (reinterpret_cast<uintptr_t>(scale) | reinterpret_cast<uintptr_t>(C)) % 8 == 0,
+                EET_ERR_INVALID_ARGUMENT, "%s: A and W must be 16-byte aligned, scale and C 8-byte", fn);
     return EET_OK;
 }
 
@@ -494,24 +588,31 @@ extern "C" int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *sc
 {
     (void)workspace;
     (void)workspace_bytes;
-    EET_REQUIRE(A && Wpacked && scale && C, EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: null pointer");
-    EET_REQUIRE(M >= 0 && N > 0 && K > 0, EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: bad sizes M=%d N=%d K=%d", M,
-                N, K);
-    EET_REQUIRE(K % 64 == 0 && N % 16 == 0, EET_ERR_UNSUPPORTED_SHAPE,
-                "eet_gemm_w8a16: need K %% 64 == 0 and N %% 16 == 0, got K=%d N=%d", K, N);
-    EET_REQUIRE((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Wpacked)) % 16 == 0 &&
-                    (reinterpret_cast<uintptr_t>(scale) | reinterpret_cast<uintptr_t>(C)) % 8 == 0,
-                EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: A and W must be 16-byte aligned, scale and C 8-byte");
+    if (int rc = check_gemm_args("eet_gemm_w8a16", A, Wpacked, scale, C, M, N, K))
+        return rc;
     if (M == 0)
         return EET_OK;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (M <= 32) {
-        SmallMConfig cfg = pick_small_m(M, N, K);
-        if (M <= 8)
-            return dispatch_small_m<1>(cfg, A, Wpacked, scale, C, M, N, K, st);
-        if (M <= 16)
-            return dispatch_small_m<2>(cfg, A, Wpacked, scale, C, M, N, K, st);
-        return dispatch_small_m<4>(cfg, A, Wpacked, scale, C, M, N, K, st);
-    }
-    return eet_gemm_w8a16_large_m(A, Wpacked, scale, C, M, N, K, st);
+    return run_gemm(GemmArgs{static_cast<const _Float16 *>(A), static_cast<const u32x4 *>(Wpacked),
+                             static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(C), M, N, K, nullptr,
+                             kEpiNone, static_cast<hipStream_t>(stream)});
+}
+
+extern "C" int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, void *C, int M, int N,
+                                    int K, int epilogue, const void *residual, void *stream)
+{
+    if (int rc = check_gemm_args("eet_gemm_w8a16_fused", A, Wpacked, scale, C, M, N, K))
+        return rc;
+    EET_REQUIRE(epilogue == EET_EPILOGUE_NONE || epilogue == EET_EPILOGUE_RESIDUAL || epilogue == EET_EPILOGUE_SWIGLU,
+                EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16_fused: unknown epilogue %d", epilogue);
+    EET_REQUIRE((epilogue == EET_EPILOGUE_RESIDUAL) == (residual != nullptr), EET_ERR_INVALID_ARGUMENT,
+                "eet_gemm_w8a16_fused: residual must be given exactly for EET_EPILOGUE_RESIDUAL");
+    EET_REQUIRE(residual == nullptr || reinterpret_cast<uintptr_t>(residual) % 8 == 0, EET_ERR_INVALID_ARGUMENT,
+                "eet_gemm_w8a16_fused: residual must be 8-byte aligned");
+    EET_REQUIRE(epilogue != EET_EPILOGUE_SWIGLU || N % 32 == 0, EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_gemm_w8a16_fused: the SwiGLU epilogue needs N %% 32 == 0 (gate/up tile pairs), got N=%d", N);
+    if (M == 0)
+        return EET_OK;
+    return run_gemm(GemmArgs{static_cast<const _Float16 *>(A), static_cast<const u32x4 *>(Wpacked),
+                             static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(C), M, N, K,
+                             static_cast<const _Float16 *>(residual), epilogue, static_cast<hipStream_t>(stream)});
 }

@@ -102,9 +102,25 @@ def _check_vec(name, v, N):
                            f"got {v.dtype} {tuple(v.shape)} on {v.device}")
 
 
-def _gemm(a, w, scale, out, M, N, K):
-    check(lib().eet_gemm_w8a16(a.data_ptr(), w.data_ptr(), scale.data_ptr(), out.data_ptr(), M, N, K, None, 0,
-                               _stream()), "eet_gemm_w8a16")
+EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
+
+
+def _gemm(a, w, scale, out, M, N, K, epilogue=EPI_NONE, residual=None):
+    check(lib().eet_gemm_w8a16_fused(a.data_ptr(), w.data_ptr(), scale.data_ptr(), out.data_ptr(), M, N, K,
+                                     epilogue, residual.data_ptr() if residual is not None else None, _stream()),
+          "eet_gemm_w8a16_fused")
+
+
+def interleave_gate_up(gate_w, gate_s, up_w, up_s):
+    """Merge two packed [K, N] weights (and their scales) tile by tile:
+    16-channel tile 2i of the result is gate tile i, tile 2i+1 is up tile i.
+    In the packed layout a tile is K*16 contiguous bytes."""
+    K, N = gate_w.shape
+    g = gate_w.reshape(N // 16, K * 16)
+    u = up_w.reshape(N // 16, K * 16)
+    w = torch.stack((g, u), 1).reshape(K, 2 * N).contiguous()
+    s = torch.stack((gate_s.reshape(N // 16, 16), up_s.reshape(N // 16, 16)), 1).reshape(2 * N).contiguous()
+    return w, s
 
 
 def _rmsnorm(x, gamma, out, M, N, eps):
@@ -231,8 +247,8 @@ class _MmhaInt8:
                                     self.v_cache.data_ptr(), cbuf.data_ptr(), _ptr(alibi), _ptr(pad), B, H, dh,
                                     self.step, self.t_cap, ws.data_ptr(), ws.numel() * 4, _stream()),
                   "eet_mmha_decode")
-        _gemm(cbuf, self.o_w, self.o_s, out, M, hidden, self.inner)
-        check(L.eet_residual_add(out.data_ptr(), x.data_ptr(), M, hidden, _stream()), "eet_residual_add")
+        # output projection with the residual add (csrc/op/llama_mmha.cpp:428-462) in its epilogue
+        _gemm(cbuf, self.o_w, self.o_s, out, M, hidden, self.inner, EPI_RESIDUAL, x)
         self._keep = (x, pad, alibi)  # inputs of kernels still in flight
         return out[: M * hidden].view(B, S, hidden)
 
@@ -283,6 +299,8 @@ class GatedFeedForwardNetworkInt8:
             Intermediate_0_weights, Intermediate_0_scale, Intermediate_1_weights, Intermediate_1_scale,
             Output_weights, Output_scale, layernorm_weights)
         self.cache_name = ffn_cache_name
+        # gate and up merged tile by tile so that one launch computes both and applies SwiGLU
+        self.w01, self.s01 = interleave_gate_up(self.w0, self.s0, self.w1, self.s1)
 
     def forward(self, input, pre_layernorm, add_residual):
         desc = self.desc
@@ -300,16 +318,15 @@ class GatedFeedForwardNetworkInt8:
         cap = desc.batch_size * max(desc.max_seq_len, 1)
         xn = workspaces.get("layernorm_tensor", cap * hidden, f16, dev)
         act = workspaces.get("ffn_inner_act", cap * self.d_ff, f16, dev)
-        lin = workspaces.get("ffn_inner_linear", cap * self.d_ff, f16, dev)
         out = workspaces.get(self.cache_name, cap * hidden, f16, dev)
-        L = lib()
         _rmsnorm(x, self.gamma, xn, M, hidden, desc.layernorm_eps)
-        _gemm(xn, self.w0, self.s0, act, M, self.d_ff, hidden)
-        _gemm(xn, self.w1, self.s1, lin, M, self.d_ff, hidden)
-        check(L.eet_swiglu(act.data_ptr(), lin.data_ptr(), M, self.d_ff, _stream()), "eet_swiglu")
-        _gemm(act, self.w2, self.s2, out, M, hidden, self.d_ff)
+        # fc1, fc2 and gated_act (gated_ffn_int8.cpp:253-301, 168-179) in one launch
+        _gemm(xn, self.w01, self.s01, act, M, 2 * self.d_ff, hidden, EPI_SWIGLU)
+        # fc3 with add_input_bias_layernorm's residual add (:303-357) in its epilogue
         if add_residual:
-            check(L.eet_residual_add(out.data_ptr(), x.data_ptr(), M, hidden, _stream()), "eet_residual_add")
+            _gemm(act, self.w2, self.s2, out, M, hidden, self.d_ff, EPI_RESIDUAL, x)
+        else:
+            _gemm(act, self.w2, self.s2, out, M, hidden, self.d_ff)
         self._keep = x
         return out[: M * hidden].view(B, S, hidden)
 

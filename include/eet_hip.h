@@ -93,6 +93,22 @@ int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *scale, void *
                    int M, int N, int K, void *workspace, size_t workspace_bytes,
                    void *stream);
 
+/* The same GEMM with a fused epilogue.
+ *   EET_EPILOGUE_NONE      C[M][N] as above.
+ *   EET_EPILOGUE_RESIDUAL  C[M][N] = half(A.W) + residual[M][N] (fp16 add): the
+ *       GEMM followed by add_bias_input_kernel with bias == nullptr, as at
+ *       csrc/op/llama_mmha.cpp:428-462 and csrc/op/gated_ffn_int8.cpp:303-357.
+ *   EET_EPILOGUE_SWIGLU    Wpacked / scale hold gate and up interleaved by
+ *       16-channel tile (tile 2i = gate tile i, tile 2i+1 = up tile i; N =
+ *       2 * d_ff); C[M][N/2] = up * gate / (1 + exp(-gate)): the two GEMMs and
+ *       gated_act_kernel of csrc/op/gated_ffn_int8.cpp:253-301, 168-179 in one
+ *       launch.  In the packed layout a 16-channel tile is one contiguous run of
+ *       K*16 bytes, so interleaving is a row-wise merge of the two packed matrices.
+ * residual must be NULL unless the epilogue is EET_EPILOGUE_RESIDUAL. */
+enum { EET_EPILOGUE_NONE = 0, EET_EPILOGUE_RESIDUAL = 1, EET_EPILOGUE_SWIGLU = 2 };
+int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, void *C,
+                         int M, int N, int K, int epilogue, const void *residual, void *stream);
+
 /* Masked multi-head decode attention for one new token per sequence.
  *   q, k, v   [B][H][dh] half; with qkv_stride != 0 they are rows of a fused
  *             buffer: element (b, h, d) at base[b * qkv_stride + h * dh + d]

@@ -109,3 +109,14 @@ def test_alibi_caller_matches_oracle():
     assert np.allclose(decoder.alibi_slopes(40), O.alibi_slopes(40))
     m = decoder.alibi_mask(8, 6).numpy()
     assert np.array_equal(np.nan_to_num(m, neginf=-1), np.nan_to_num(O.alibi_mask(8, 6), neginf=-1))
+
+
+def test_fused_argument_errors():
+    from eet_amd._lib import lib
+    buf = np.zeros(4096, np.uint8)
+    p = buf.ctypes.data
+    L = lib()
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 7, None, None) == -1          # unknown epilogue
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 1, None, None) == -1          # residual missing
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 0, p, None) == -1             # residual without the epilogue
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 48, 64, 2, None, None) == -2          # odd tile count

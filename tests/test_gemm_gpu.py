@@ -115,3 +115,43 @@ def test_full_size_linearity(gpu):
     c2 = gemm(a.to(gpu), p, (s * 2).to(gpu), M, N, K).float().cpu()
     # exact, except where the smaller result is an fp16 subnormal (one subnormal step = 2^-24)
     assert ((c2 - ca * 2).abs() <= 2.0 ** -24).all()
+
+
+def fused(a, wp, s, M, N, K, epi, residual=None):
+    from eet_amd._lib import check, lib
+    from gpu_util import stream
+    n_out = N // 2 if epi == 2 else N
+    c = torch.empty(M, n_out, dtype=torch.float16, device=a.device)
+    check(lib().eet_gemm_w8a16_fused(a.data_ptr(), wp.data_ptr(), s.data_ptr(), c.data_ptr(), M, N, K, epi,
+                                     residual.data_ptr() if residual is not None else None, stream()))
+    return c
+
+
+@pytest.mark.parametrize("M", [1, 8, 13, 32, 70, 300])
+def test_residual_epilogue(gpu, M):
+    K, N = 1024, 528
+    x, u, p, s = make(M, K, N, 40 + M)
+    res = torch.randn(M, N, generator=torch.Generator().manual_seed(M)).half()
+    xd, pd, sd, rd = x.to(gpu), p.to(gpu), s.to(gpu), res.to(gpu)
+    got = fused(xd, pd, sd, M, N, K, 1, rd).cpu()
+    plain = gemm(xd, pd, sd, M, N, K).cpu()
+    assert torch.equal(got, (plain + res))          # fp16 add of the rounded product, bit for bit
+    want = O.residual_add(O.dequant_matmul(x.numpy(), u.numpy(), s.numpy()), res.numpy())
+    assert_close(got.numpy(), want, rtol=1e-2, atol=2e-3)
+
+
+@pytest.mark.parametrize("M,K,F", [(1, 256, 64), (8, 4096, 11008), (16, 512, 208), (32, 512, 704), (100, 256, 96),
+                                   (260, 512, 1376)])
+def test_swiglu_epilogue(gpu, M, K, F):
+    from eet_amd.ops import interleave_gate_up
+    g = torch.Generator().manual_seed(F + M)
+    x = torch.randn(M, K, generator=g).half()
+    wg = (torch.randn(K, F, generator=g) * 0.02).half()
+    wu = (torch.randn(K, F, generator=g) * 0.02).half()
+    ug, pg, sg = eet_amd.quant_weights(wg, torch.int8, True)
+    uu, pu, su = eet_amd.quant_weights(wu, torch.int8, True)
+    w01, s01 = interleave_gate_up(pg, sg, pu, su)
+    got = fused(x.to(gpu), w01.to(gpu), s01.to(gpu), M, 2 * F, K, 2).cpu().numpy()
+    want = O.swiglu(O.dequant_matmul(x.numpy(), ug.numpy(), sg.numpy()),
+                    O.dequant_matmul(x.numpy(), uu.numpy(), su.numpy()))
+    assert_close(got, want, rtol=1e-2, atol=1e-3)

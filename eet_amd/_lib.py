@@ -24,7 +24,8 @@ SIGNATURES = {
     "eet_gemm_w8a16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _vp]),
     "eet_gemm_w8a16_fused": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "eet_mmha_decode_workspace": (_sz, [_i, _i, _i, _i]),
-    "eet_mmha_decode": (_i, [_vp, _vp, _vp, _l, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "eet_mmha_decode": (_i, [_vp, _vp, _vp, _l, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
+    "eet_rope_table": (_i, [_vp, _i, _i, _vp]),
     "eet_rmsnorm": (_i, [_vp, _vp, _vp, _i, _i, _f, _vp]),
     "eet_qkv_split": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "eet_swiglu": (_i, [_vp, _vp, _i, _i, _vp]),

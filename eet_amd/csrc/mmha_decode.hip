@@ -77,6 +77,26 @@ __device__ __forceinline__ float block_reduce(float v, bool is_max, float *scrat
     return r;
 }
 
+// NeoX rotary on one 8-element slice.  x holds elements d = 8*sub .. 8*sub+7 of
+// a head row, y the slice DH/2 away; rope_row is [cos(DH/2) | sin(DH/2)] for the
+// position.  fp32 math, one rounding to fp16 (csrc/core/common.cuh:209-225).
+template <int DH>
+__device__ __forceinline__ u32x4 rotate8(const u32x4 &x, const u32x4 &y, int sub, const float *rope_row)
+{
+    constexpr int LPR = DH / 8;
+    const bool lower = sub < LPR / 2;
+    const int i0 = (sub % (LPR / 2)) * 8;
+    const half8 hx = __builtin_bit_cast(half8, x), hy = __builtin_bit_cast(half8, y);
+    half8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float c = rope_row[i0 + e], sn = rope_row[DH / 2 + i0 + e];
+        const float a = (float)hx[e], b = (float)hy[e];
+        o[e] = (_Float16)(lower ? a * c - b * sn : a * c + b * sn);
+    }
+    return __builtin_bit_cast(u32x4, o);
+}
+
 // DH: head size.  LPR = DH/8 lanes cover one row with one 16-byte load each.
 // PREFILL = false: one query per (b, h), rows [0, step).
 // PREFILL = true : blockIdx.x also runs over the S = step prompt positions;
@@ -87,7 +107,7 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_new, const _Float16 *__restrict__ v_new,
     long qkv_stride, _Float16 *__restrict__ k_cache, _Float16 *__restrict__ v_cache, _Float16 *__restrict__ ctx,
     const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, float *__restrict__ partial, int H,
-    int step_or_S, int T_cap, int nsplit, float scale)
+    int step_or_S, int T_cap, int nsplit, float scale, const float *__restrict__ rope_row)
 {
     constexpr int LPR = DH / 8;            // lanes per row
     constexpr int RPB = kThreads / LPR;    // rows in flight per pass of the block
@@ -121,21 +141,34 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
     const int n = max(0, t1 - t0);
 
     // Append the new token's k, v (row step-1).  Only the workgroup that owns
-    // that row writes it, then reads it back like any other row.
+    // that row writes it, then reads it back like any other row.  With a rotary
+    // row given, k is rotated on the way in (pairs d, d + DH/2).
     if (k_new != nullptr && step - 1 >= t0 && step - 1 < t1) {
         if (tid < LPR) {
-            *reinterpret_cast<uint4 *>(kc + (size_t)(step - 1) * DH + tid * 8) =
-                *reinterpret_cast<const uint4 *>(k_new + qoff + tid * 8);
+            u32x4 kx = *reinterpret_cast<const u32x4 *>(k_new + qoff + tid * 8);
+            if (rope_row != nullptr) {
+                const u32x4 ky = *reinterpret_cast<const u32x4 *>(k_new + qoff + (tid ^ (LPR / 2)) * 8);
+                kx = rotate8<DH>(kx, ky, tid, rope_row);
+            }
+            *reinterpret_cast<u32x4 *>(kc + (size_t)(step - 1) * DH + tid * 8) = kx;
         } else if (tid < 2 * LPR) {
             const int s2 = tid - LPR;
-            *reinterpret_cast<uint4 *>(vc + (size_t)(step - 1) * DH + s2 * 8) =
-                *reinterpret_cast<const uint4 *>(v_new + qoff + s2 * 8);
+            *reinterpret_cast<u32x4 *>(vc + (size_t)(step - 1) * DH + s2 * 8) =
+                *reinterpret_cast<const u32x4 *>(v_new + qoff + s2 * 8);
         }
         __threadfence();
     }
     __syncthreads();
 
-    const u32x4 qv = *reinterpret_cast<const u32x4 *>(q + qoff + sub * 8);
+    u32x4 qv = *reinterpret_cast<const u32x4 *>(q + qoff + sub * 8);
+    if (!PREFILL && rope_row != nullptr) {
+        u32x4 qy;
+        qy.x = __shfl_xor(qv.x, LPR / 2, 64);
+        qy.y = __shfl_xor(qv.y, LPR / 2, 64);
+        qy.z = __shfl_xor(qv.z, LPR / 2, 64);
+        qy.w = __shfl_xor(qv.w, LPR / 2, 64);
+        qv = rotate8<DH>(qv, qy, sub, rope_row);
+    }
 
     // Phase 1: logits of rows [t0, t1).
     float lmax = -INFINITY;
@@ -252,7 +285,7 @@ int pick_nsplit(int BH, int step)
 template <int DH>
 int launch(const void *q, const void *k, const void *v, long qkv_stride, void *kc, void *vc, void *ctx,
            const void *alibi, const int64_t *pad, int B, int H, int step, int T_cap, void *ws, int nsplit,
-           hipStream_t st)
+           const float *rope_row, hipStream_t st)
 {
     const float scale = (float)(_Float16)(1.0f / sqrtf((float)DH));
     dim3 grid(B * H, nsplit);
@@ -261,7 +294,7 @@ int launch(const void *q, const void *k, const void *v, long qkv_stride, void *k
                        static_cast<const _Float16 *>(v), qkv_stride, static_cast<_Float16 *>(kc),
                        static_cast<_Float16 *>(vc), static_cast<_Float16 *>(ctx),
                        static_cast<const _Float16 *>(alibi), pad, static_cast<float *>(ws), H, step, T_cap, nsplit,
-                       scale);
+                       scale, rope_row);
     EET_HIP_CHECK(hipGetLastError());
     if (nsplit > 1) {
         hipLaunchKernelGGL((mmha_decode_merge_kernel<DH>), dim3(B * H), dim3(DH), 0, st,
@@ -280,7 +313,7 @@ int launch_prefill(const void *q, const void *kc, const void *vc, void *ctx, con
                        static_cast<const _Float16 *>(q), nullptr, nullptr, 0L,
                        static_cast<_Float16 *>(const_cast<void *>(kc)),
                        static_cast<_Float16 *>(const_cast<void *>(vc)), static_cast<_Float16 *>(ctx),
-                       static_cast<const _Float16 *>(alibi), pad, nullptr, H, S, T_cap, 1, scale);
+                       static_cast<const _Float16 *>(alibi), pad, nullptr, H, S, T_cap, 1, scale, nullptr);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
@@ -310,6 +343,32 @@ extern "C" int eet_prefill_attention(const void *q, const void *k_cache, const v
     }
 }
 
+namespace {
+// table[t][i] = cos(t / 10000^(2i/dh)), table[t][dh/2 + i] = sin(...), fp32
+// (csrc/core/common.cuh:176-180).
+__global__ void rope_table_kernel(float *table, int T, int dh)
+{
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= T * (dh / 2))
+        return;
+    const int t = idx / (dh / 2), i = idx % (dh / 2);
+    const float ang = (float)t / powf(10000.0f, (float)(2 * i) / (float)dh);
+    table[(size_t)t * dh + i] = cosf(ang);
+    table[(size_t)t * dh + dh / 2 + i] = sinf(ang);
+}
+}  // namespace
+
+extern "C" int eet_rope_table(float *table, int T, int dh, void *stream)
+{
+    EET_REQUIRE(table != nullptr, EET_ERR_INVALID_ARGUMENT, "eet_rope_table: null pointer");
+    EET_REQUIRE(T > 0 && dh > 0 && dh % 2 == 0, EET_ERR_INVALID_ARGUMENT, "eet_rope_table: bad sizes T=%d dh=%d", T, dh);
+    const int n = T * (dh / 2);
+    hipLaunchKernelGGL(rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), table,
+                       T, dh);
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
 extern "C" size_t eet_mmha_decode_workspace(int B, int H, int dh, int step)
 {
     if (B <= 0 || H <= 0 || dh <= 0 || step <= 0)
@@ -320,7 +379,8 @@ extern "C" size_t eet_mmha_decode_workspace(int B, int H, int dh, int step)
 
 extern "C" int eet_mmha_decode(const void *q, const void *k, const void *v, long qkv_stride, void *k_cache,
                                void *v_cache, void *ctx, const void *alibi, const int64_t *pad, int B, int H,
-                               int dh, int step, int T_cap, void *workspace, size_t workspace_bytes, void *stream)
+                               int dh, int step, int T_cap, const float *rope_cos_sin, void *workspace,
+                               size_t workspace_bytes, void *stream)
 {
     EET_REQUIRE(q && k_cache && v_cache && ctx, EET_ERR_INVALID_ARGUMENT, "eet_mmha_decode: null pointer");
     EET_REQUIRE((k == nullptr) == (v == nullptr), EET_ERR_INVALID_ARGUMENT,
@@ -333,6 +393,8 @@ extern "C" int eet_mmha_decode(const void *q, const void *k, const void *v, long
                 "eet_mmha_decode: head size %d not supported (32, 64, 128)", dh);
     EET_REQUIRE(qkv_stride >= 0 && qkv_stride % 8 == 0, EET_ERR_INVALID_ARGUMENT,
                 "eet_mmha_decode: qkv_stride must be a non-negative multiple of 8");
+    EET_REQUIRE(rope_cos_sin == nullptr || k != nullptr, EET_ERR_INVALID_ARGUMENT,
+                "eet_mmha_decode: a rotary row needs the new k, v (it rotates q and the appended k)");
     const int ns = pick_nsplit(B * H, step);
     const size_t need = eet_mmha_decode_workspace(B, H, dh, step);
     EET_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), EET_ERR_WORKSPACE,
@@ -341,12 +403,12 @@ extern "C" int eet_mmha_decode(const void *q, const void *k, const void *v, long
     switch (dh) {
         case 32:
             return launch<32>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, workspace,
-                              ns, st);
+                              ns, rope_cos_sin, st);
         case 64:
             return launch<64>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, workspace,
-                              ns, st);
+                              ns, rope_cos_sin, st);
         default:
             return launch<128>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap,
-                               workspace, ns, st);
+                               workspace, ns, rope_cos_sin, st);
     }
 }

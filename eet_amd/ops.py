@@ -130,6 +130,20 @@ def _rmsnorm(x, gamma, out, M, N, eps):
 # ----------------------------------------------------------------------------
 # attention ops
 # ----------------------------------------------------------------------------
+_rope_tables = {}
+
+
+def _rope_table(T, dh, device):
+    """fp32 [T, dh] table (cos | sin per position), built once per (T, dh, device)."""
+    key = (T, dh, str(device))
+    t = _rope_tables.get(key)
+    if t is None:
+        t = torch.empty(T, dh, dtype=torch.float32, device=device)
+        check(lib().eet_rope_table(t.data_ptr(), T, dh, _stream()), "eet_rope_table")
+        _rope_tables[key] = t
+    return t
+
+
 class _MmhaInt8:
     """Shared body of LlamaMmha (rotary) and BaichuanMmha (ALiBi)."""
 
@@ -168,6 +182,7 @@ class _MmhaInt8:
         self.v_cache = torch.zeros_like(self.k_cache)
         self.step = 1
         self.first_batch = 0
+        self.rope_table = _rope_table(self.t_cap, self.dh, dev) if self._rope else None
 
     def forward(self, input, pre_padding_len, reorder_state, pre_layernorm, add_residual, first_pass,
                 relative_attention_bias=_EMPTY):
@@ -220,10 +235,11 @@ class _MmhaInt8:
         out = workspaces.get("self_mask_attn_cache", desc.batch_size * max(desc.max_seq_len, 1) * hidden, f16, dev)
         _rmsnorm(x, self.gamma, xn, M, hidden, desc.layernorm_eps)
         _gemm(xn, self.qkv_w, self.qkv_s, qkv, M, 3 * self.inner, hidden)
-        check(L.eet_qkv_split(qkv.data_ptr(), qbuf.data_ptr(), self.k_cache.data_ptr(), self.v_cache.data_ptr(),
-                              B, S, H, dh, 1 if self._rope else 0, time_step, t0, self.t_cap, _stream()),
-              "eet_qkv_split")
         if first_pass:
+            # split (+ rotary at position s) and write K, V rows [0, S) of the cache
+            check(L.eet_qkv_split(qkv.data_ptr(), qbuf.data_ptr(), self.k_cache.data_ptr(),
+                                  self.v_cache.data_ptr(), B, S, H, dh, 1 if self._rope else 0, -1, 0, self.t_cap,
+                                  _stream()), "eet_qkv_split")
             alibi = None
             if bias is not None:
                 # [H, S, S] mask whose row i holds slope*j for j <= i: its last row is the whole table
@@ -242,10 +258,13 @@ class _MmhaInt8:
                 alibi = bias.to(f16).contiguous()
             need = L.eet_mmha_decode_workspace(B, H, dh, self.step)
             ws = workspaces.get("mmha_ws", max(need // 4, 1), torch.float32, dev)
-            # k, v already sit in the cache (written by eet_qkv_split), so no append here
-            check(L.eet_mmha_decode(qbuf.data_ptr(), None, None, 0, self.k_cache.data_ptr(),
+            # q, k, v are read straight from the fused GEMM output; the kernel rotates q and k
+            # (rotary op only) and appends k, v at row step-1
+            base, hd = qkv.data_ptr(), self.inner
+            rope = self.rope_table.data_ptr() + (self.step - 1) * dh * 4 if self._rope else None
+            check(L.eet_mmha_decode(base, base + 2 * hd, base + 4 * hd, 3 * hd, self.k_cache.data_ptr(),
                                     self.v_cache.data_ptr(), cbuf.data_ptr(), _ptr(alibi), _ptr(pad), B, H, dh,
-                                    self.step, self.t_cap, ws.data_ptr(), ws.numel() * 4, _stream()),
+                                    self.step, self.t_cap, rope, ws.data_ptr(), ws.numel() * 4, _stream()),
                   "eet_mmha_decode")
         # output projection with the residual add (csrc/op/llama_mmha.cpp:428-462) in its epilogue
         _gemm(cbuf, self.o_w, self.o_s, out, M, hidden, self.inner, EPI_RESIDUAL, x)

@@ -117,6 +117,11 @@ int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, 
  *   alibi     NULL or [H][step] half, added to the scaled logits
  *   pad       NULL or [B] int64: rows t < pad[b] get zero weight
  *   ctx       [B][H*dh] half
+ *   rope_cos_sin  NULL, or the row of the eet_rope_table table for this token's
+ *             position (dh floats: cos[dh/2] | sin[dh/2]); q and the appended k
+ *             are then rotated NeoX-style in the kernel, which stands in for
+ *             fused_QKV_neox_rotary_transpose (csrc/core/self_add_bias.cu:369-403)
+ *             at decode time.  Needs k, v != NULL.
  *   workspace eet_mmha_decode_workspace(B, H, dh, step) bytes of device memory
  * softmax denominator carries the reference's + 1e-6.
  * Replaces masked_attention_dispatch (csrc/core/attention_dispatch.cu:888-928)
@@ -125,7 +130,12 @@ size_t eet_mmha_decode_workspace(int B, int H, int dh, int step);
 int eet_mmha_decode(const void *q, const void *k, const void *v, long qkv_stride,
                     void *k_cache, void *v_cache, void *ctx, const void *alibi,
                     const int64_t *pad, int B, int H, int dh, int step, int T_cap,
-                    void *workspace, size_t workspace_bytes, void *stream);
+                    const float *rope_cos_sin, void *workspace, size_t workspace_bytes,
+                    void *stream);
+
+/* table[t][0 .. dh/2) = cos(t / 10000^(2i/dh)), table[t][dh/2 .. dh) = sin(...),
+ * t in [0, T): the rotary coefficients of csrc/core/common.cuh:176-180 in fp32. */
+int eet_rope_table(float *table, int T, int dh, void *stream);
 
 /* out[M][N] = x * rsqrt(mean(x^2) + eps) * gamma.  Replaces RMSnorm
  * (csrc/core/layer_norm.cu:580-625). */

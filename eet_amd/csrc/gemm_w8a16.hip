@@ -66,6 +66,7 @@ template <int NT, int RG, int U>
 struct Batch {
     u32x4 w[U][NT];
     u32x4 a[U][RG];
+    u32x4 gam[U];  // RMSnorm weights of the lane's piece (only with the RMSnorm prologue)
 };
 
 // Activation loads are issued so that a wavefront reads whole 128-byte lines:
@@ -74,9 +75,9 @@ struct Batch {
 // operand straight from the row-major matrix instead costs 16 half-used lines
 // per instruction and measured 1.4 us (M = 8) to 2.5 us (M = 16) on a 4 us
 // kernel.
-template <int NT, int RG, int WAVES, int U>
+template <int NT, int RG, int WAVES, int U, bool RMS>
 __device__ __forceinline__ void load_batch(Batch<NT, RG, U> &b, const u32x4 *const (&wbase)[NT],
-                                           const u32x4 *const (&abase)[RG], int kt)
+                                           const u32x4 *const (&abase)[RG], const u32x4 *gbase, int kt)
 {
     // All weight loads (HBM latency) go out first, then the activation loads
     // (L2 hits); loads return in issue order.
@@ -91,6 +92,11 @@ __device__ __forceinline__ void load_batch(Batch<NT, RG, U> &b, const u32x4 *con
 #pragma unroll
         for (int r = 0; r < RG; ++r)
             b.a[u][r] = abase[r][(kt + u * WAVES) * 8];
+    if (RMS) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            b.gam[u] = gbase[(kt + u * WAVES) * 8];
+    }
     __builtin_amdgcn_sched_barrier(0);
 }
 
@@ -98,9 +104,9 @@ __device__ __forceinline__ void load_batch(Batch<NT, RG, U> &b, const u32x4 *con
 // wavefront-private LDS slab: lane (g, j) of operand half h needs piece
 // 2*g + h of row j.  Piece p of row jr is kept at slot jr*8 + (p ^ jr), which
 // makes both the 16-byte writes and the 16-byte reads bank-conflict free.
-template <int NT, int RG, int U>
+template <int NT, int RG, int U, bool RMS>
 __device__ __forceinline__ void mma_batch(const Batch<NT, RG, U> &b, floatx4 (&acc)[NT][(RG + 1) / 2],
-                                          u32x4 *slab, int lane)
+                                          u32x4 *slab, int lane, float (&ss)[RG])
 {
     constexpr int MT = (RG + 1) / 2;
     const int g = lane >> 4, j = lane & 15;
@@ -109,8 +115,22 @@ __device__ __forceinline__ void mma_batch(const Batch<NT, RG, U> &b, floatx4 (&a
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
-        for (int r = 0; r < RG; ++r)
-            slab[(u * RG + r) * 64 + wslot] = b.a[u][r];
+        for (int r = 0; r < RG; ++r) {
+            u32x4 piece = b.a[u][r];
+            if (RMS) {
+                // RMSnorm prologue: accumulate sum(x^2) of the row and feed x * gamma
+                // (fp16) to the MFMA; 1/rms is applied to the fp32 sum in the epilogue.
+                const half8 x = __builtin_bit_cast(half8, piece);
+                const half2v x0 = __builtin_shufflevector(x, x, 0, 1), x1 = __builtin_shufflevector(x, x, 2, 3);
+                const half2v x2 = __builtin_shufflevector(x, x, 4, 5), x3 = __builtin_shufflevector(x, x, 6, 7);
+                ss[r] = __builtin_amdgcn_fdot2(x0, x0, ss[r], false);
+                ss[r] = __builtin_amdgcn_fdot2(x1, x1, ss[r], false);
+                ss[r] = __builtin_amdgcn_fdot2(x2, x2, ss[r], false);
+                ss[r] = __builtin_amdgcn_fdot2(x3, x3, ss[r], false);
+                piece = __builtin_bit_cast(u32x4, x * __builtin_bit_cast(half8, b.gam[u]));
+            }
+            slab[(u * RG + r) * 64 + wslot] = piece;
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -138,10 +158,13 @@ __device__ __forceinline__ void mma_batch(const Batch<NT, RG, U> &b, floatx4 (&a
 }
 
 // NT: n-tiles per workgroup.  RG: groups of 8 activation rows (M <= 8 * RG).
-template <int NT, int RG, int WAVES, int U>
+// RMS: RMSnorm prologue compiled in (it costs ~20-30 registers, so the plain
+// GEMM is a separate instantiation).
+template <int NT, int RG, int WAVES, int U, bool RMS>
 __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
-    _Float16 *__restrict__ C, int M, int N, int K, const _Float16 *__restrict__ residual, int epi)
+    _Float16 *__restrict__ C, int M, int N, int K, const _Float16 *__restrict__ residual, int epi,
+    const _Float16 *__restrict__ rms_gamma, float rms_eps)
 {
     constexpr int MT = (RG + 1) / 2;
     const int lane = threadIdx.x & 63;
@@ -182,6 +205,13 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         abase[r] = reinterpret_cast<const u32x4 *>(A + (size_t)m * K) + (lane & 7);
     }
 
+    constexpr bool rms = RMS;
+    const u32x4 *gbase = rms ? reinterpret_cast<const u32x4 *>(rms_gamma) + (lane & 7) : nullptr;
+    float ss[RG];
+#pragma unroll
+    for (int r = 0; r < RG; ++r)
+        ss[r] = 0.f;
+
     // This wavefront's k-tiles are wave, wave + WAVES, ...; they are taken in
     // batches of U with the next batch's loads in flight while the current one
     // is multiplied (two register buffers).
@@ -192,25 +222,25 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     {
         Batch<NT, RG, U> b0, b1;
         if (nbatch > 0)
-            load_batch<NT, RG, WAVES, U>(b0, wbase, abase, kt);
+            load_batch<NT, RG, WAVES, U, RMS>(b0, wbase, abase, gbase, kt);
         int i = 0;
         for (; i + 2 <= nbatch; i += 2) {
-            load_batch<NT, RG, WAVES, U>(b1, wbase, abase, kt + STEP);
-            mma_batch<NT, RG, U>(b0, acc, slab, lane);
+            load_batch<NT, RG, WAVES, U, RMS>(b1, wbase, abase, gbase, kt + STEP);
+            mma_batch<NT, RG, U, RMS>(b0, acc, slab, lane, ss);
             if (i + 2 < nbatch)
-                load_batch<NT, RG, WAVES, U>(b0, wbase, abase, kt + 2 * STEP);
-            mma_batch<NT, RG, U>(b1, acc, slab, lane);
+                load_batch<NT, RG, WAVES, U, RMS>(b0, wbase, abase, gbase, kt + 2 * STEP);
+            mma_batch<NT, RG, U, RMS>(b1, acc, slab, lane, ss);
             kt += 2 * STEP;
         }
         if (i < nbatch) {
-            mma_batch<NT, RG, U>(b0, acc, slab, lane);
+            mma_batch<NT, RG, U, RMS>(b0, acc, slab, lane, ss);
             kt += STEP;
         }
     }
     for (; kt < ktiles; kt += WAVES) {
         Batch<NT, RG, 1> b;
-        load_batch<NT, RG, WAVES, 1>(b, wbase, abase, kt);
-        mma_batch<NT, RG, 1>(b, acc, slab, lane);
+        load_batch<NT, RG, WAVES, 1, RMS>(b, wbase, abase, gbase, kt);
+        mma_batch<NT, RG, 1, RMS>(b, acc, slab, lane, ss);
     }
 
     // Epilogue operands (per-channel scales, residual rows) are requested before
@@ -236,6 +266,21 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         }
     }
 
+    // RMSnorm prologue: each wavefront's share of sum(x^2) per row.  Lanes
+    // 8*q .. 8*q+7 hold pieces of row 8*r + q.
+    __shared__ float rowss[WAVES][RG * 8];
+    if (rms) {
+#pragma unroll
+        for (int r = 0; r < RG; ++r) {
+            float v = ss[r];
+            v += __shfl_xor(v, 1, 64);
+            v += __shfl_xor(v, 2, 64);
+            v += __shfl_xor(v, 4, 64);
+            if ((lane & 7) == 0)
+                rowss[wave][r * 8 + (lane >> 3)] = v;
+        }
+    }
+
     // Cross-wavefront reduction.  acc[t][mt][r] of lane (g, j) is the product
     // for channel 16*(nt0+t) + 4*g + r and row 16*mt + j.
     __syncthreads();  // every wavefront is done with its activation slab
@@ -257,6 +302,15 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     for (int unit = wave; unit < units; unit += WAVES, ++idx) {
         const int mt = unit % MT;
         const int m = mt * 16 + j;
+        float inv = 1.0f;
+        if (rms) {
+            const int row = min(m, RG * 8 - 1);
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w)
+                tot += rowss[w][row];
+            inv = rsqrtf(tot / (float)K + rms_eps);
+        }
         if (epi == kEpiSwiglu) {
             const int t = 2 * (unit / MT);
             const floatx4 sg = tile_sum(t * MT + mt), su = tile_sum((t + 1) * MT + mt);
@@ -265,8 +319,8 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
                 half4 o;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float gate = (float)(_Float16)(sg[r] * (float)sc0[idx][r]);
-                    const float up = (float)(_Float16)(su[r] * (float)sc1[idx][r]);
+                    const float gate = (float)(_Float16)(sg[r] * (float)sc0[idx][r] * inv);
+                    const float up = (float)(_Float16)(su[r] * (float)sc1[idx][r] * inv);
                     o[r] = (_Float16)(up * gate / (1.0f + __expf(-gate)));
                 }
                 const int n = ((nt0 + t) / 2) * 16 + 4 * g;
@@ -280,7 +334,7 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
                 half4 o;
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    o[r] = (_Float16)(s[r] * (float)sc0[idx][r]);
+                    o[r] = (_Float16)(s[r] * (float)sc0[idx][r] * inv);
                 if (epi == kEpiResidual)
                     o = o + res[idx];  // fp16 add of the rounded product, like the separate kernel
                 *reinterpret_cast<half4 *>(C + (size_t)m * N + n) = o;
@@ -301,16 +355,18 @@ struct GemmArgs {
     int M, N, K;
     const _Float16 *residual;
     int epi;
+    const _Float16 *rms_gamma;  // non-null: RMSnorm prologue (small-M kernel only)
+    float rms_eps;
     hipStream_t st;
 };
 
-template <int NT, int RG, int WAVES, int U>
+template <int NT, int RG, int WAVES, int U, bool RMS>
 int launch_small_m(const GemmArgs &a)
 {
     const int ntiles = a.N / 16;
     dim3 grid((ntiles + NT - 1) / NT), block(WAVES * 64);
-    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U>), grid, block, 0, a.st, a.A, a.Wp, a.scale, a.C, a.M,
-                       a.N, a.K, a.residual, a.epi);
+    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U, RMS>), grid, block, 0, a.st, a.A, a.Wp, a.scale, a.C, a.M,
+                       a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
@@ -331,12 +387,26 @@ int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a)
 #define EET_CASE(NT_, W_, U_)                                      \
     if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_) {         \
         if constexpr (small_m_fits(NT_, RG, W_, U_))               \
-            return launch_small_m<NT_, RG, W_, U_>(a);             \
+            return launch_small_m<NT_, RG, W_, U_, false>(a);      \
+    }
+#define EET_CASE_RMS(NT_, W_, U_)                                  \
+    if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_) {         \
+        if constexpr (small_m_fits(NT_, RG, W_, U_))               \
+            return launch_small_m<NT_, RG, W_, U_, true>(a);       \
+    }
+    if (a.rms_gamma != nullptr) {
+        // the launch shapes pick_small_m can return
+        EET_CASE_RMS(1, 8, 2) EET_CASE_RMS(1, 16, 2) EET_CASE_RMS(1, 16, 1)
+        EET_CASE_RMS(2, 8, 2) EET_CASE_RMS(2, 8, 1) EET_CASE_RMS(3, 8, 1)
+        return eet::fail(EET_ERR_INVALID_ARGUMENT,
+                         "eet_gemm_w8a16_fused: no RMSnorm-prologue kernel for nt=%d waves=%d u=%d", cfg.nt,
+                         cfg.waves, cfg.u);
     }
     EET_CASE(1, 4, 4) EET_CASE(1, 8, 4) EET_CASE(1, 16, 4) EET_CASE(1, 8, 2) EET_CASE(1, 16, 2) EET_CASE(1, 16, 1)
     EET_CASE(2, 4, 2) EET_CASE(2, 8, 2) EET_CASE(2, 16, 2) EET_CASE(2, 8, 4) EET_CASE(2, 16, 1) EET_CASE(2, 8, 1)
     EET_CASE(3, 8, 2) EET_CASE(3, 16, 2) EET_CASE(3, 16, 1) EET_CASE(3, 8, 1)
     EET_CASE(4, 4, 2) EET_CASE(4, 8, 2) EET_CASE(4, 8, 1) EET_CASE(4, 16, 1)
+#undef EET_CASE_RMS
 #undef EET_CASE
     return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no small-M kernel for nt=%d waves=%d u=%d (M=%d)",
                      cfg.nt, cfg.waves, cfg.u, a.M);
@@ -594,11 +664,12 @@ extern "C" int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *sc
         return EET_OK;
     return run_gemm(GemmArgs{static_cast<const _Float16 *>(A), static_cast<const u32x4 *>(Wpacked),
                              static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(C), M, N, K, nullptr,
-                             kEpiNone, static_cast<hipStream_t>(stream)});
+                             kEpiNone, nullptr, 0.f, static_cast<hipStream_t>(stream)});
 }
 
 extern "C" int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, void *C, int M, int N,
-                                    int K, int epilogue, const void *residual, void *stream)
+                                    int K, int epilogue, const void *residual, const void *rms_gamma, float rms_eps,
+                                    void *stream)
 {
     if (int rc = check_gemm_args("eet_gemm_w8a16_fused", A, Wpacked, scale, C, M, N, K))
         return rc;
@@ -610,9 +681,14 @@ extern "C" int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const vo
                 "eet_gemm_w8a16_fused: residual must be 8-byte aligned");
     EET_REQUIRE(epilogue != EET_EPILOGUE_SWIGLU || N % 32 == 0, EET_ERR_UNSUPPORTED_SHAPE,
                 "eet_gemm_w8a16_fused: the SwiGLU epilogue needs N %% 32 == 0 (gate/up tile pairs), got N=%d", N);
+    EET_REQUIRE(rms_gamma == nullptr || (M <= 32 && reinterpret_cast<uintptr_t>(rms_gamma) % 16 == 0),
+                EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_gemm_w8a16_fused: the RMSnorm prologue is available for M <= 32 only (M=%d) and needs a "
+                "16-byte aligned gamma", M);
     if (M == 0)
         return EET_OK;
     return run_gemm(GemmArgs{static_cast<const _Float16 *>(A), static_cast<const u32x4 *>(Wpacked),
                              static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(C), M, N, K,
-                             static_cast<const _Float16 *>(residual), epilogue, static_cast<hipStream_t>(stream)});
+                             static_cast<const _Float16 *>(residual), epilogue,
+                             static_cast<const _Float16 *>(rms_gamma), rms_eps, static_cast<hipStream_t>(stream)});
 }

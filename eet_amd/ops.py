@@ -105,9 +105,13 @@ def _check_vec(name, v, N):
 EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 
 
-def _gemm(a, w, scale, out, M, N, K, epilogue=EPI_NONE, residual=None):
+RMS_FUSE_MAX_M = 32     # the RMSnorm prologue exists in the small-M kernel only
+
+
+def _gemm(a, w, scale, out, M, N, K, epilogue=EPI_NONE, residual=None, rms_gamma=None, rms_eps=0.0):
     check(lib().eet_gemm_w8a16_fused(a.data_ptr(), w.data_ptr(), scale.data_ptr(), out.data_ptr(), M, N, K,
-                                     epilogue, residual.data_ptr() if residual is not None else None, _stream()),
+                                     epilogue, residual.data_ptr() if residual is not None else None,
+                                     rms_gamma.data_ptr() if rms_gamma is not None else None, rms_eps, _stream()),
           "eet_gemm_w8a16_fused")
 
 
@@ -233,8 +237,13 @@ class _MmhaInt8:
         qbuf = workspaces.get("q_buf", desc.batch_size * max(desc.max_seq_len, 1) * self.inner, f16, dev)
         cbuf = workspaces.get("context_buf", desc.batch_size * max(desc.max_seq_len, 1) * self.inner, f16, dev)
         out = workspaces.get("self_mask_attn_cache", desc.batch_size * max(desc.max_seq_len, 1) * hidden, f16, dev)
-        _rmsnorm(x, self.gamma, xn, M, hidden, desc.layernorm_eps)
-        _gemm(xn, self.qkv_w, self.qkv_s, qkv, M, 3 * self.inner, hidden)
+        if M <= RMS_FUSE_MAX_M:
+            # RMSnorm folded into the GEMM's activation load
+            _gemm(x, self.qkv_w, self.qkv_s, qkv, M, 3 * self.inner, hidden, EPI_NONE, None, self.gamma,
+                  desc.layernorm_eps)
+        else:
+            _rmsnorm(x, self.gamma, xn, M, hidden, desc.layernorm_eps)
+            _gemm(xn, self.qkv_w, self.qkv_s, qkv, M, 3 * self.inner, hidden)
         if first_pass:
             # split (+ rotary at position s) and write K, V rows [0, S) of the cache
             check(L.eet_qkv_split(qkv.data_ptr(), qbuf.data_ptr(), self.k_cache.data_ptr(),
@@ -338,9 +347,14 @@ class GatedFeedForwardNetworkInt8:
         xn = workspaces.get("layernorm_tensor", cap * hidden, f16, dev)
         act = workspaces.get("ffn_inner_act", cap * self.d_ff, f16, dev)
         out = workspaces.get(self.cache_name, cap * hidden, f16, dev)
-        _rmsnorm(x, self.gamma, xn, M, hidden, desc.layernorm_eps)
-        # fc1, fc2 and gated_act (gated_ffn_int8.cpp:253-301, 168-179) in one launch
-        _gemm(xn, self.w01, self.s01, act, M, 2 * self.d_ff, hidden, EPI_SWIGLU)
+        # fc1, fc2 and gated_act (gated_ffn_int8.cpp:253-301, 168-179) in one launch; at decode
+        # sizes the RMSnorm (:112) rides in the same launch
+        if M <= RMS_FUSE_MAX_M:
+            _gemm(x, self.w01, self.s01, act, M, 2 * self.d_ff, hidden, EPI_SWIGLU, None, self.gamma,
+                  desc.layernorm_eps)
+        else:
+            _rmsnorm(x, self.gamma, xn, M, hidden, desc.layernorm_eps)
+            _gemm(xn, self.w01, self.s01, act, M, 2 * self.d_ff, hidden, EPI_SWIGLU)
         # fc3 with add_input_bias_layernorm's residual add (:303-357) in its epilogue
         if add_residual:
             _gemm(act, self.w2, self.s2, out, M, hidden, self.d_ff, EPI_RESIDUAL, x)

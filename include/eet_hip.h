@@ -104,10 +104,17 @@ int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *scale, void *
  *       gated_act_kernel of csrc/op/gated_ffn_int8.cpp:253-301, 168-179 in one
  *       launch.  In the packed layout a 16-channel tile is one contiguous run of
  *       K*16 bytes, so interleaving is a row-wise merge of the two packed matrices.
- * residual must be NULL unless the epilogue is EET_EPILOGUE_RESIDUAL. */
+ * residual must be NULL unless the epilogue is EET_EPILOGUE_RESIDUAL.
+ * RMSnorm prologue (rms_gamma != NULL, M <= 32): A is the un-normalised input
+ * and the result is that of eet_rmsnorm(A, rms_gamma, rms_eps) followed by the
+ * GEMM -- the RMSnorm + GEMM pairs at csrc/op/llama_mmha.cpp:222-227 and
+ * csrc/op/gated_ffn_int8.cpp:112-116 in one launch.  The kernel multiplies
+ * x * gamma in fp16 on the way in, accumulates sum(x^2) per row, and applies
+ * rsqrt(mean + eps) to the fp32 accumulator. */
 enum { EET_EPILOGUE_NONE = 0, EET_EPILOGUE_RESIDUAL = 1, EET_EPILOGUE_SWIGLU = 2 };
 int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, void *C,
-                         int M, int N, int K, int epilogue, const void *residual, void *stream);
+                         int M, int N, int K, int epilogue, const void *residual,
+                         const void *rms_gamma, float rms_eps, void *stream);
 
 /* Masked multi-head decode attention for one new token per sequence.
  *   q, k, v   [B][H][dh] half; with qkv_stride != 0 they are rows of a fused

@@ -118,7 +118,8 @@ def test_fused_argument_errors():
     buf = np.zeros(4096, np.uint8)
     p = buf.ctypes.data
     L = lib()
-    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 7, None, None) == -1          # unknown epilogue
-    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 1, None, None) == -1          # residual missing
-    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 0, p, None) == -1             # residual without the epilogue
-    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 48, 64, 2, None, None) == -2          # odd tile count
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 7, None, None, 0.0, None) == -1          # unknown epilogue
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 1, None, None, 0.0, None) == -1          # residual missing
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 0, p, None, 0.0, None) == -1             # residual without the epilogue
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 48, 64, 2, None, None, 0.0, None) == -2          # odd tile count
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 64, 32, 64, 0, None, p, 1e-6, None) == -2       # RMSnorm prologue, M > 32

@@ -117,13 +117,14 @@ def test_full_size_linearity(gpu):
     assert ((c2 - ca * 2).abs() <= 2.0 ** -24).all()
 
 
-def fused(a, wp, s, M, N, K, epi, residual=None):
+def fused(a, wp, s, M, N, K, epi, residual=None, gamma=None, eps=0.0):
     from eet_amd._lib import check, lib
     from gpu_util import stream
     n_out = N // 2 if epi == 2 else N
     c = torch.empty(M, n_out, dtype=torch.float16, device=a.device)
     check(lib().eet_gemm_w8a16_fused(a.data_ptr(), wp.data_ptr(), s.data_ptr(), c.data_ptr(), M, N, K, epi,
-                                     residual.data_ptr() if residual is not None else None, stream()))
+                                     residual.data_ptr() if residual is not None else None,
+                                     gamma.data_ptr() if gamma is not None else None, eps, stream()))
     return c
 
 
@@ -155,3 +156,51 @@ def test_swiglu_epilogue(gpu, M, K, F):
     want = O.swiglu(O.dequant_matmul(x.numpy(), ug.numpy(), sg.numpy()),
                     O.dequant_matmul(x.numpy(), uu.numpy(), su.numpy()))
     assert_close(got, want, rtol=1e-2, atol=1e-3)
+
+
+@pytest.mark.parametrize("M,K,N,epi", [(1, 256, 64, 0), (8, 4096, 12288, 0), (8, 4096, 22016, 2), (16, 1024, 176, 0),
+                                       (32, 512, 96, 2), (5, 11008, 4096, 1)])
+def test_rmsnorm_prologue(gpu, M, K, N, epi):
+    """RMSnorm folded into the GEMM against the fp32 composition rmsnorm -> GEMM (-> epilogue).
+
+    The fused kernel rounds x * gamma to fp16 and applies 1/rms to the fp32 sum; the unfused path
+    rounds x * gamma / rms to fp16.  Both carry one fp16 rounding per activation, at different
+    places, so the comparison is against the composition with NO intermediate rounding, with the
+    absolute tolerance doubled to 2e-3 for that one rounding (relative stays 1e-2)."""
+    from eet_amd.ops import interleave_gate_up
+    g = torch.Generator().manual_seed(M + K + N)
+    x = (torch.randn(M, K, generator=g) * 1.7).half()
+    gamma = (1 + 0.1 * torch.randn(K, generator=g)).half()
+    eps = 1e-6
+    x32 = x.numpy().astype(np.float32)
+    xn = x32 / np.sqrt((x32 * x32).mean(-1, keepdims=True) + eps) * gamma.numpy().astype(np.float32)
+
+    def mm(u, s):
+        return xn @ (u.numpy().astype(np.float32) * s.numpy().astype(np.float32)[None, :])
+    if epi == 2:
+        F = N // 2
+        ug, pg, sg = eet_amd.quant_weights((torch.randn(K, F, generator=g) * 0.02).half(), torch.int8, True)
+        uu, pu, su = eet_amd.quant_weights((torch.randn(K, F, generator=g) * 0.02).half(), torch.int8, True)
+        p, s = interleave_gate_up(pg, sg, pu, su)
+        gate, up = mm(ug, sg), mm(uu, su)
+        want = up * gate / (1 + np.exp(-gate))
+        res = None
+    else:
+        u, p, s = eet_amd.quant_weights((torch.randn(K, N, generator=g) * 0.02).half(), torch.int8, True)
+        want = mm(u, s)
+        res = torch.randn(M, N, generator=g).half() if epi == 1 else None
+        if epi == 1:
+            want = want + res.numpy().astype(np.float32)
+    rd = res.to(gpu) if res is not None else None
+    got = fused(x.to(gpu), p.to(gpu), s.to(gpu), M, N, K, epi, rd, gamma.to(gpu), eps).cpu().numpy()
+    # the SwiGLU epilogue adds the fp16 roundings of gate and up (as the separate kernels have them)
+    atol = 3e-3 if epi == 2 else 2e-3
+    assert_close(got, want, rtol=1e-2, atol=atol)
+    # and the unfused path (eet_rmsnorm then the GEMM) agrees with the same reference
+    from eet_amd._lib import check, lib
+    from gpu_util import stream
+    xd, gd = x.to(gpu), gamma.to(gpu)
+    xnd = torch.empty_like(xd)
+    check(lib().eet_rmsnorm(xd.data_ptr(), gd.data_ptr(), xnd.data_ptr(), M, K, eps, stream()))
+    got2 = fused(xnd, p.to(gpu), s.to(gpu), M, N, K, epi, rd).cpu().numpy()
+    assert_close(got2, want, rtol=1e-2, atol=atol)

@@ -188,6 +188,86 @@ def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed):
             "note": "greedy decode, random-init weights, random token ids; lm_head and embedding are fp16 torch ops"}
 
 
+MFMA_FP16_PEAK_TFLOPS = 2500.0   # MI355X published dense fp16 MFMA peak
+
+
+def prefill_gemm_bench(torch, eet, lib, dev, iters=10):
+    """BASELINE config 3: Baichuan-13B-shaped prefill GEMMs, M = 2048 tokens, on the MFMA kernel.
+    Reports TFLOP/s = 2*M*N*K / t and the fraction of the fp16 MFMA peak."""
+    M, hidden, d_ff = 2048, 5120, 13696
+    g = torch.Generator(device=dev).manual_seed(21)
+    out = {}
+    st = torch.cuda.current_stream()
+    for name, K, N in (("qkv", hidden, 3 * hidden), ("o", hidden, hidden), ("gate", hidden, d_ff),
+                       ("down", d_ff, hidden)):
+        w = (torch.randn(K, N, generator=g, device=dev) * 0.02).half()
+        q, s = eet.quant_weights_torch(w, "ref128")
+        p = eet.pack_weights_torch(q)
+        del w, q
+        a = torch.randn(M, K, generator=g, device=dev).half()
+        c = torch.empty(M, N, dtype=torch.float16, device=dev)
+        args = (a.data_ptr(), p.data_ptr(), s.data_ptr(), c.data_ptr(), M, N, K, None, 0, st.cuda_stream)
+        for _ in range(2):
+            if lib.eet_gemm_w8a16(*args):
+                raise RuntimeError(lib.eet_last_error().decode())
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(st)
+        for _ in range(iters):
+            lib.eet_gemm_w8a16(*args)
+        e1.record(st)
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e-3 / iters
+        tf = 2.0 * M * N * K / t / 1e12
+        out[f"{name} M={M} K={K} N={N}"] = {"us": round(t * 1e6, 1), "TFLOP/s": round(tf, 1),
+                                            "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4)}
+    return out
+
+
+def attention_bench(torch, lib, dev, iters=20):
+    """Isolated masked decode attention at the config 4 (LLaMA-7B, B=8) and config 5 (Baichuan-13B,
+    B=32, ALiBi) shapes: GB/s over the algorithmic bytes 2*step*B*H*dh*2 + 6*B*H*dh*2 (+ 2*H*step)."""
+    out = {}
+    st = torch.cuda.current_stream()
+    for name, B, H, step, alibi in (("llama7b B=8 step=1088", 8, 32, 1088, False),
+                                    ("baichuan13b B=32 step=2176 alibi", 32, 40, 2176, True)):
+        dh, cap = 128, step + 1
+        g = torch.Generator(device=dev).manual_seed(step)
+        # several caches in rotation so that the rows come from HBM, not the 256 MB Infinity Cache
+        per = 2 * B * H * cap * dh * 2
+        ncache = max(2, int(600e6 // per) + 1)
+        caches = [(torch.randn(B, H, cap, dh, generator=g, device=dev).half(),
+                   torch.randn(B, H, cap, dh, generator=g, device=dev).half()) for _ in range(ncache)]
+        q, k, v = [torch.randn(B, H, dh, generator=g, device=dev).half() for _ in range(3)]
+        ctx = torch.empty(B, H * dh, dtype=torch.float16, device=dev)
+        bias = (torch.rand(H, step, generator=g, device=dev) * 8).half() if alibi else None
+        need = lib.eet_mmha_decode_workspace(B, H, dh, step)
+        ws = torch.empty(max(need // 4, 1), dtype=torch.float32, device=dev)
+
+        def call(i):
+            kc, vc = caches[i % ncache]
+            rc = lib.eet_mmha_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), 0, kc.data_ptr(), vc.data_ptr(),
+                                     ctx.data_ptr(), bias.data_ptr() if alibi else None, None, B, H, dh, step, cap,
+                                     None, ws.data_ptr(), ws.numel() * 4, st.cuda_stream)
+            if rc:
+                raise RuntimeError(lib.eet_last_error().decode())
+        for i in range(ncache):
+            call(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(st)
+        for i in range(iters):
+            call(i)
+        e1.record(st)
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e-3 / iters
+        nbytes = 2 * step * B * H * dh * 2 + 6 * B * H * dh * 2 + (2 * H * step if alibi else 0)
+        out[name] = {"us": round(t * 1e6, 1), "GB/s": round(nbytes / t / 1e9, 1),
+                     "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4), "bytes": nbytes}
+        del caches
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -283,6 +363,10 @@ def main():
                     "pct_peak": round(100 * b * n / s / 1e9 / HBM_PEAK_GBS, 2)}
         result["gemm_by_m"] = sweep
         result[f"gemm_by_shape_M{M}"] = per_shape
+
+    if not args.no_sweep:
+        result["prefill_gemm_config3"] = prefill_gemm_bench(torch, eet, L, dev)
+        result["decode_attention"] = attention_bench(torch, L, dev)
 
     if args.gen > 0:
         result["decode"] = decode_bench(torch, eet, weights, dev, args.batch, args.prompt, args.gen, seed=7)

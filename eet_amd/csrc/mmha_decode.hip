@@ -15,9 +15,13 @@
 // (the reference runs one block per head); every workgroup produces an
 // un-normalised partial (max, sum, acc[dh]) and a second small kernel merges
 // them.  With nsplit == 1 the first kernel writes the context itself.
+// Inside a workgroup every group of dh/8 lanes streams its own rows with a
+// running softmax, K and V rows requested together several rows deep; there
+// is no per-launch limit on step.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <cstdlib>
 
 #include "common.h"
 
@@ -28,7 +32,6 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
-constexpr int kMaxChunk = 2048;  // logits of one workgroup's time range, kept in LDS
 
 __device__ __forceinline__ float dot8(const u32x4 &a, const u32x4 &b)
 {
@@ -102,7 +105,7 @@ __device__ __forceinline__ u32x4 rotate8(const u32x4 &x, const u32x4 &y, int sub
 // PREFILL = true : blockIdx.x also runs over the S = step prompt positions;
 //   query i of q[B][H][S][dh] attends rows [0, i] and writes ctx[b][i][h*dh..]
 //   (the causal prompt pass, one workgroup per query row; nsplit is 1).
-template <int DH, bool PREFILL>
+template <int DH, bool PREFILL, int UN>
 __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_new, const _Float16 *__restrict__ v_new,
     long qkv_stride, _Float16 *__restrict__ k_cache, _Float16 *__restrict__ v_cache, _Float16 *__restrict__ ctx,
@@ -110,10 +113,9 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
     int step_or_S, int T_cap, int nsplit, float scale, const float *__restrict__ rope_row)
 {
     constexpr int LPR = DH / 8;            // lanes per row
-    constexpr int RPB = kThreads / LPR;    // rows in flight per pass of the block
-    __shared__ float logits[kMaxChunk];
-    __shared__ float red[kThreads / 64];
+    constexpr int RPB = kThreads / LPR;    // row streams of the block (one per group of LPR lanes)
     __shared__ float accs[RPB][DH + 1];
+    __shared__ float stream_m[RPB], stream_l[RPB];
 
     const int split = blockIdx.y;
     const int bh = PREFILL ? blockIdx.x / step_or_S : blockIdx.x;
@@ -171,76 +173,73 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
         qv = rotate8<DH>(qv, qy, sub, rope_row);
     }
 
-    // Phase 1: logits of rows [t0, t1).
-    float lmax = -INFINITY;
-    for (int r0 = 0; r0 < n; r0 += RPB * 4) {
-        u32x4 kv[4];
+    // Every group of LPR lanes walks its own stream of rows (rs, rs + RPB, ...)
+    // with a running softmax (max m, sum l, un-normalised acc): K and V rows are
+    // requested together, UN rows deep, and nothing synchronises the workgroup
+    // until the streams are merged at the end.
+    float m_run = -INFINITY, l_run = 0.f;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int r0 = rs; r0 < n; r0 += RPB * UN) {
+        u32x4 kv[UN], vv[UN];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int r = r0 + u * RPB + rs;
+        for (int u = 0; u < UN; ++u) {
+            const int r = r0 + u * RPB;
             if (r < n)
                 kv[u] = (r == r_last)
                             ? knew
                             : load_row16<!PREFILL>(reinterpret_cast<const u32x4 *>(kc + (size_t)(t0 + r) * DH) + sub);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int r = r0 + u * RPB + rs;
-            float d = (r < n) ? dot8(qv, kv[u]) : 0.f;
-            d = group_sum<LPR>(d) * scale;
-            if (r < n) {
-                if (alibi)
-                    d += (float)alibi[(size_t)h * alibi_ld + t0 + r];
-                if (sub == 0)
-                    logits[r] = d;
-                lmax = fmaxf(lmax, d);
-            }
-        }
-    }
-    lmax = block_reduce(lmax, true, red);  // also orders the logits[] writes
-
-    // Phase 2: un-normalised weights and their sum.
-    float lsum = 0.f;
-    for (int r = tid; r < n; r += kThreads) {
-        float p = __expf(logits[r] - lmax);
-        logits[r] = p;
-        lsum += p;
-    }
-    lsum = block_reduce(lsum, false, red);
-
-    // Phase 3: acc = sum_t p_t * v_t.
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int r0 = 0; r0 < n; r0 += RPB * 4) {
-        u32x4 vv[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int r = r0 + u * RPB + rs;
+        for (int u = 0; u < UN; ++u) {
+            const int r = r0 + u * RPB;
             if (r < n)
                 vv[u] = (r == r_last)
                             ? vnew
                             : load_row16<!PREFILL>(reinterpret_cast<const u32x4 *>(vc + (size_t)(t0 + r) * DH) + sub);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int r = r0 + u * RPB + rs;
+        for (int u = 0; u < UN; ++u) {
+            const int r = r0 + u * RPB;  // the same for all LPR lanes of a group
+            float d = (r < n) ? dot8(qv, kv[u]) : 0.f;
+            d = group_sum<LPR>(d) * scale;
             if (r < n) {
-                const float p = logits[r];
+                if (alibi)
+                    d += (float)alibi[(size_t)h * alibi_ld + t0 + r];
+                const float m_new = fmaxf(m_run, d);
+                const float c = __expf(m_run - m_new);  // 0 on the first row (m_run = -inf)
+                const float p = __expf(d - m_new);
+                l_run = l_run * c + p;
                 const half8 hv = __builtin_bit_cast(half8, vv[u]);
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    acc[e] += p * (float)hv[e];
+                    acc[e] = acc[e] * c + p * (float)hv[e];
+                m_run = m_new;
             }
         }
     }
+
+    // Merge the RPB streams of the workgroup.
 #pragma unroll
     for (int e = 0; e < 8; ++e)
         accs[rs][sub * 8 + e] = acc[e];
+    if (sub == 0) {
+        stream_m[rs] = m_run;
+        stream_l[rs] = l_run;
+    }
     __syncthreads();
     if (tid < DH) {
-        float s = 0.f;
+        float lmax = -INFINITY;
 #pragma unroll 4
         for (int r = 0; r < RPB; ++r)
-            s += accs[r][tid];
+            lmax = fmaxf(lmax, stream_m[r]);
+        float s = 0.f, lsum = 0.f;
+#pragma unroll 4
+        for (int r = 0; r < RPB; ++r) {
+            const float mr = stream_m[r];
+            const float w = (mr == -INFINITY) ? 0.f : __expf(mr - lmax);
+            lsum += w * stream_l[r];
+            s += w * accs[r][tid];
+        }
         if (nsplit == 1) {
             // n == 0 (everything padded away) gives 0 / 1e-6 = 0.
             ctx[coff + tid] = (_Float16)(s / (lsum + 1e-6f));
@@ -276,14 +275,17 @@ __global__ __launch_bounds__(DH) void mmha_decode_merge_kernel(const float *__re
 
 int pick_nsplit(int BH, int step)
 {
-    // enough workgroups for ~4 per CU, at least 64 rows each, and no more rows
-    // per workgroup than the LDS logits array holds
-    int want = (1024 + BH - 1) / BH;
-    int by_rows = (step + 63) / 64;
+    static const int forced = [] {
+        const char *e = std::getenv("EET_MMHA_NSPLIT");  // tuning override
+        return e ? atoi(e) : 0;
+    }();
+    if (forced > 0)
+        return forced;
+    // Measured on MI355X (B*H = 256 at step ~1100 and B*H = 1280 at step ~2200):
+    // up to ~4096 workgroups, but no fewer than 256 rows each.
+    int want = (4096 + BH - 1) / BH;
+    int by_rows = step / 256;
     int ns = want < by_rows ? want : by_rows;
-    int need = (step + kMaxChunk - 1) / kMaxChunk;
-    if (ns < need)
-        ns = need;
     return ns < 1 ? 1 : ns;
 }
 
@@ -294,7 +296,12 @@ int launch(const void *q, const void *k, const void *v, long qkv_stride, void *k
 {
     const float scale = (float)(_Float16)(1.0f / sqrtf((float)DH));
     dim3 grid(B * H, nsplit);
-    hipLaunchKernelGGL((mmha_decode_split_kernel<DH, false>), grid, dim3(kThreads), 0, st,
+    static const int unroll = [] {
+        const char *e = std::getenv("EET_MMHA_UNROLL");
+        return e ? atoi(e) : 8;
+    }();
+    auto kern = (unroll == 4) ? mmha_decode_split_kernel<DH, false, 4> : mmha_decode_split_kernel<DH, false, 8>;
+    hipLaunchKernelGGL(kern, grid, dim3(kThreads), 0, st,
                        static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(k),
                        static_cast<const _Float16 *>(v), qkv_stride, static_cast<_Float16 *>(kc),
                        static_cast<_Float16 *>(vc), static_cast<_Float16 *>(ctx),
@@ -314,7 +321,7 @@ int launch_prefill(const void *q, const void *kc, const void *vc, void *ctx, con
                    int B, int H, int S, int T_cap, hipStream_t st)
 {
     const float scale = (float)(_Float16)(1.0f / sqrtf((float)DH));
-    hipLaunchKernelGGL((mmha_decode_split_kernel<DH, true>), dim3((unsigned)(B * H * S), 1), dim3(kThreads), 0, st,
+    hipLaunchKernelGGL((mmha_decode_split_kernel<DH, true, 4>), dim3((unsigned)(B * H * S), 1), dim3(kThreads), 0, st,
                        static_cast<const _Float16 *>(q), nullptr, nullptr, 0L,
                        static_cast<_Float16 *>(const_cast<void *>(kc)),
                        static_cast<_Float16 *>(const_cast<void *>(vc)), static_cast<_Float16 *>(ctx),
@@ -336,8 +343,6 @@ extern "C" int eet_prefill_attention(const void *q, const void *k_cache, const v
                 "eet_prefill_attention: bad sizes B=%d H=%d S=%d T_cap=%d", B, H, S, T_cap);
     EET_REQUIRE(dh == 32 || dh == 64 || dh == 128, EET_ERR_UNSUPPORTED_SHAPE,
                 "eet_prefill_attention: head size %d not supported (32, 64, 128)", dh);
-    EET_REQUIRE(S <= kMaxChunk, EET_ERR_UNSUPPORTED_SHAPE, "eet_prefill_attention: prompt length %d exceeds %d", S,
-                kMaxChunk);
     EET_REQUIRE((long long)B * H * S < (1LL << 31), EET_ERR_UNSUPPORTED_SHAPE,
                 "eet_prefill_attention: B*H*S too large");
     hipStream_t st = static_cast<hipStream_t>(stream);

@@ -29,7 +29,18 @@ def _ptr(t):
 
 
 def _stream():
-    return torch.cuda.current_stream().cuda_stream
+    return _StreamScope.handle if _StreamScope.handle is not None else torch.cuda.current_stream().cuda_stream
+
+
+class _StreamScope:
+    """Looks torch's current stream up once per op call instead of once per kernel."""
+    handle = None
+
+    def __enter__(self):
+        _StreamScope.handle = torch.cuda.current_stream().cuda_stream
+
+    def __exit__(self, *a):
+        _StreamScope.handle = None
 
 
 # ----------------------------------------------------------------------------
@@ -190,6 +201,12 @@ class _MmhaInt8:
 
     def forward(self, input, pre_padding_len, reorder_state, pre_layernorm, add_residual, first_pass,
                 relative_attention_bias=_EMPTY):
+        with _StreamScope():
+            return self._forward(input, pre_padding_len, reorder_state, pre_layernorm, add_residual, first_pass,
+                                 relative_attention_bias)
+
+    def _forward(self, input, pre_padding_len, reorder_state, pre_layernorm, add_residual, first_pass,
+                 relative_attention_bias):
         # pre_layernorm / add_residual are accepted and ignored exactly as in the
         # reference: it always normalises first and always adds the input back
         # (csrc/op/llama_mmha.cpp:136, 222, 462).
@@ -331,6 +348,10 @@ class GatedFeedForwardNetworkInt8:
         self.w01, self.s01 = interleave_gate_up(self.w0, self.s0, self.w1, self.s1)
 
     def forward(self, input, pre_layernorm, add_residual):
+        with _StreamScope():
+            return self._forward(input, pre_layernorm, add_residual)
+
+    def _forward(self, input, pre_layernorm, add_residual):
         desc = self.desc
         if input.dtype != torch.float16 or input.dim() != 3 or input.shape[2] != desc.hidden_units:
             raise RuntimeError(f"[EET][ERROR] GatedFeedForwardNetworkInt8: input must be fp16 [B, S, "

@@ -71,7 +71,7 @@ def test_device_entry_points_validate_before_launch():
     assert L.eet_qkv_split(p, p, p, p, 1, 4, 1, 128, 1, -1, 6, 8, None) == -1  # rows past the cache end
     assert L.eet_swiglu(p, p, 1, 12, None) == -2
     assert L.eet_residual_add(p, None, 1, 16, None) == -1
-    assert L.eet_prefill_attention(p, p, p, p, None, None, 1, 1, 4096, 128, 4096, None) == -2
+    assert L.eet_prefill_attention(p, p, p, p, None, None, 1, 1, 4096, 96, 4096, None) == -2
 
 
 def test_python_api_errors():

@@ -179,7 +179,11 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     constexpr int kSlabVec = U * RG * 64;                      // u32x4 per wavefront
     constexpr int kStageBytes = WAVES * kSlabVec * 16;
     constexpr int kRedBytes = WAVES * NT * MT * 64 * 16;
-    __shared__ __attribute__((aligned(16))) unsigned char lds[kStageBytes > kRedBytes ? kStageBytes : kRedBytes];
+    // The two regions share memory only when both together would not fit 64 KiB
+    // (sharing costs a second barrier in the epilogue).
+    constexpr bool kAlias = kStageBytes + kRedBytes > 65536;
+    constexpr int kLdsBytes = kAlias ? (kStageBytes > kRedBytes ? kStageBytes : kRedBytes) : kStageBytes + kRedBytes;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[kLdsBytes];
     u32x4 *slab = reinterpret_cast<u32x4 *>(lds) + wave * kSlabVec;
 
     floatx4 acc[NT][MT];
@@ -204,6 +208,32 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         int m = min(8 * r + (lane >> 3), M - 1);
         abase[r] = reinterpret_cast<const u32x4 *>(A + (size_t)m * K) + (lane & 7);
     }
+
+    // Epilogue operands (per-channel scales, residual rows) are requested first
+    // of all, so that a miss in L2 is long over when the epilogue needs them.
+    // An output unit is
+    // one (n-tile, m-tile) product, or for the SwiGLU epilogue the pair of
+    // adjacent n-tiles (gate, up) of one m-tile.
+    constexpr int kMaxUnits = (NT * MT + WAVES - 1) / WAVES;
+    const int units = (epi == kEpiSwiglu) ? (NT / 2) * MT : NT * MT;
+    half4 sc0[kMaxUnits], sc1[kMaxUnits], res[kMaxUnits];
+    {
+        int idx = 0;
+        for (int unit = wave; unit < units; unit += WAVES, ++idx) {
+            const int mt = unit % MT;
+            const int t = (epi == kEpiSwiglu) ? 2 * (unit / MT) : unit / MT;
+            const int nt = min(nt0 + t, ntiles - 1);
+            sc0[idx] = *reinterpret_cast<const half4 *>(scale + nt * 16 + 4 * g);
+            if (epi == kEpiSwiglu)
+                sc1[idx] = *reinterpret_cast<const half4 *>(scale + min(nt + 1, ntiles - 1) * 16 + 4 * g);
+            if (epi == kEpiResidual) {
+                const int m = min(mt * 16 + j, M - 1);
+                res[idx] = *reinterpret_cast<const half4 *>(residual + (size_t)m * N + nt * 16 + 4 * g);
+            }
+        }
+    }
+
+    __builtin_amdgcn_sched_barrier(0);
 
     constexpr bool rms = RMS;
     const u32x4 *gbase = rms ? reinterpret_cast<const u32x4 *>(rms_gamma) + (lane & 7) : nullptr;
@@ -243,29 +273,6 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         mma_batch<NT, RG, 1, RMS>(b, acc, slab, lane, ss);
     }
 
-    // Epilogue operands (per-channel scales, residual rows) are requested before
-    // the barrier so their latency overlaps the reduction.  An output unit is
-    // one (n-tile, m-tile) product, or for the SwiGLU epilogue the pair of
-    // adjacent n-tiles (gate, up) of one m-tile.
-    constexpr int kMaxUnits = (NT * MT + WAVES - 1) / WAVES;
-    const int units = (epi == kEpiSwiglu) ? (NT / 2) * MT : NT * MT;
-    half4 sc0[kMaxUnits], sc1[kMaxUnits], res[kMaxUnits];
-    {
-        int idx = 0;
-        for (int unit = wave; unit < units; unit += WAVES, ++idx) {
-            const int mt = unit % MT;
-            const int t = (epi == kEpiSwiglu) ? 2 * (unit / MT) : unit / MT;
-            const int nt = min(nt0 + t, ntiles - 1);
-            sc0[idx] = *reinterpret_cast<const half4 *>(scale + nt * 16 + 4 * g);
-            if (epi == kEpiSwiglu)
-                sc1[idx] = *reinterpret_cast<const half4 *>(scale + min(nt + 1, ntiles - 1) * 16 + 4 * g);
-            if (epi == kEpiResidual) {
-                const int m = min(mt * 16 + j, M - 1);
-                res[idx] = *reinterpret_cast<const half4 *>(residual + (size_t)m * N + nt * 16 + 4 * g);
-            }
-        }
-    }
-
     // RMSnorm prologue: each wavefront's share of sum(x^2) per row.  Lanes
     // 8*q .. 8*q+7 hold pieces of row 8*r + q.
     __shared__ float rowss[WAVES][RG * 8];
@@ -283,8 +290,9 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
 
     // Cross-wavefront reduction.  acc[t][mt][r] of lane (g, j) is the product
     // for channel 16*(nt0+t) + 4*g + r and row 16*mt + j.
-    __syncthreads();  // every wavefront is done with its activation slab
-    floatx4 *red = reinterpret_cast<floatx4 *>(lds);  // [WAVES][NT * MT][64]
+    if (kAlias)
+        __syncthreads();  // every wavefront is done with its activation slab
+    floatx4 *red = reinterpret_cast<floatx4 *>(lds + (kAlias ? 0 : kStageBytes));  // [WAVES][NT * MT][64]
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll

@@ -316,42 +316,7 @@ int launch(const void *q, const void *k, const void *v, long qkv_stride, void *k
     return EET_OK;
 }
 
-template <int DH>
-int launch_prefill(const void *q, const void *kc, const void *vc, void *ctx, const void *alibi, const int64_t *pad,
-                   int B, int H, int S, int T_cap, hipStream_t st)
-{
-    const float scale = (float)(_Float16)(1.0f / sqrtf((float)DH));
-    hipLaunchKernelGGL((mmha_decode_split_kernel<DH, true, 4>), dim3((unsigned)(B * H * S), 1), dim3(kThreads), 0, st,
-                       static_cast<const _Float16 *>(q), nullptr, nullptr, 0L,
-                       static_cast<_Float16 *>(const_cast<void *>(kc)),
-                       static_cast<_Float16 *>(const_cast<void *>(vc)), static_cast<_Float16 *>(ctx),
-                       static_cast<const _Float16 *>(alibi), pad, nullptr, H, S, T_cap, 1, scale, nullptr);
-    EET_HIP_CHECK(hipGetLastError());
-    return EET_OK;
-}
-
 }  // namespace
-
-// Interim prompt pass: one workgroup per query row re-using the decode kernel
-// (K and V rows are re-read per query from L2).  Correct, not fast.
-extern "C" int eet_prefill_attention(const void *q, const void *k_cache, const void *v_cache, void *ctx,
-                                     const void *alibi, const int64_t *pad, int B, int H, int S, int dh, int T_cap,
-                                     void *stream)
-{
-    EET_REQUIRE(q && k_cache && v_cache && ctx, EET_ERR_INVALID_ARGUMENT, "eet_prefill_attention: null pointer");
-    EET_REQUIRE(B > 0 && H > 0 && S > 0 && S <= T_cap, EET_ERR_INVALID_ARGUMENT,
-                "eet_prefill_attention: bad sizes B=%d H=%d S=%d T_cap=%d", B, H, S, T_cap);
-    EET_REQUIRE(dh == 32 || dh == 64 || dh == 128, EET_ERR_UNSUPPORTED_SHAPE,
-                "eet_prefill_attention: head size %d not supported (32, 64, 128)", dh);
-    EET_REQUIRE((long long)B * H * S < (1LL << 31), EET_ERR_UNSUPPORTED_SHAPE,
-                "eet_prefill_attention: B*H*S too large");
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    switch (dh) {
-        case 32: return launch_prefill<32>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
-        case 64: return launch_prefill<64>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
-        default: return launch_prefill<128>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
-    }
-}
 
 namespace {
 // table[t][i] = cos(t / 10000^(2i/dh)), table[t][dh/2 + i] = sin(...), fp32

@@ -64,7 +64,10 @@ def test_swiglu_and_residual(gpu):
 
 
 @pytest.mark.parametrize("B,H,S,dh,use_pad,use_alibi", [(2, 3, 9, 128, False, False), (2, 2, 40, 64, True, False),
-                                                       (1, 4, 130, 128, False, True), (2, 2, 33, 32, True, True)])
+                                                       (1, 4, 130, 128, False, True), (2, 2, 33, 32, True, True),
+                                                       (1, 1, 1, 128, False, False), (2, 2, 64, 128, False, False),
+                                                       (2, 3, 300, 128, True, False), (1, 2, 257, 64, True, True),
+                                                       (1, 2, 1024, 128, False, False), (1, 1, 2500, 128, False, True)])
 def test_prefill_attention(gpu, B, H, S, dh, use_pad, use_alibi):
     g = torch.Generator().manual_seed(S)
     cap = S + 5
@@ -72,7 +75,7 @@ def test_prefill_attention(gpu, B, H, S, dh, use_pad, use_alibi):
     kc = torch.zeros(B, H, cap, dh).half()
     vc = torch.zeros(B, H, cap, dh).half()
     kc[:, :, :S], vc[:, :, :S] = k, v
-    pad = torch.tensor([0, 3][:B]) if use_pad else None
+    pad = torch.tensor([0, min(S - 1, 70)][:B] if B > 1 else [min(S - 1, 70)]) if use_pad else None
     bias_full = O.alibi_mask(H, S) if use_alibi else None
     want = O.prefill_attention(q.numpy(), k.numpy(), v.numpy(), pad.numpy() if use_pad else None, bias_full)
     ctx = torch.empty(B, S, H * dh, dtype=torch.float16, device=gpu)

@@ -458,8 +458,8 @@ int run_small_m(const GemmArgs &a)
 // ---------------------------------------------------------------------------
 // Large-M kernel (M > 32, prefill; fp16-MFMA bound).
 //
-// Block tile 128 (M) x 256 (N) x 64 (K), 4 wavefronts side by side along N,
-// each 128 x 64 = 8 m-tiles x 4 n-tiles of v_mfma_f32_16x16x32_f16 (128 fp32
+// Block tile 128 (M) x 256 or 128 (N) x 64 (K), 4 wavefronts side by side along N,
+// each 8 m-tiles x TN (4 or 2) n-tiles of v_mfma_f32_16x16x32_f16 (128 or 64 fp32
 // accumulator registers).  Weights: every wavefront reads its own four packed
 // tiles straight from global memory into registers -- the packed layout is
 // already the MFMA operand layout, so they never touch LDS -- and widens them
@@ -470,8 +470,9 @@ int run_small_m(const GemmArgs &a)
 // Workgroups are numbered so that the ones sharing a weight column block run
 // on the same XCD (workgroup i lands on XCD i % 8) and hit its L2.
 // ---------------------------------------------------------------------------
-constexpr int kLmBM = 128, kLmBN = 256, kLmTM = kLmBM / 16, kLmTN = 4;
+constexpr int kLmBM = 128, kLmTM = kLmBM / 16;  // the block is 128 rows x (4 wavefronts x TN n-tiles x 16) channels
 
+template <int kLmTN>
 __global__ __launch_bounds__(256) void w8a16_large_m_kernel(const _Float16 *__restrict__ A,
                                                             const u32x4 *__restrict__ Wp,
                                                             const _Float16 *__restrict__ scale,
@@ -494,7 +495,7 @@ __global__ __launch_bounds__(256) void w8a16_large_m_kernel(const _Float16 *__re
         return;
     const int n_blk = tile / m_blocks, m_blk = tile % m_blocks;
     const int m0 = m_blk * kLmBM;
-    const int nt0 = n_blk * (kLmBN / 16) + wave * kLmTN;
+    const int nt0 = n_blk * (4 * kLmTN) + wave * kLmTN;
 
     const u32x4 *wbase[kLmTN];
 #pragma unroll
@@ -532,15 +533,15 @@ __global__ __launch_bounds__(256) void w8a16_large_m_kernel(const _Float16 *__re
 
     const int rslot0 = g * 16 + (j ^ (2 * g)), rslot1 = g * 16 + (j ^ (2 * g + 1));
     for (int kt = 0; kt < ktiles; ++kt) {
-        const bool more = kt + 1 < ktiles;
-        if (more) {
+        // prefetch the next k-tile (the last iteration re-reads its own tile: no branch around the loads)
+        const int kn = min(kt + 1, ktiles - 1);
 #pragma unroll
-            for (int t = 0; t < kLmTN; ++t)
-                wnext[t] = wbase[t][(size_t)(kt + 1) * 64];
+        for (int t = 0; t < kLmTN; ++t)
+            wnext[t] = wbase[t][(size_t)kn * 64];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                areg[i] = asrc[i][(kt + 1) * 8];
-        }
+        for (int i = 0; i < 4; ++i)
+            areg[i] = asrc[i][kn * 8];
+        __builtin_amdgcn_sched_barrier(0);
         half8 w0[kLmTN], w1[kLmTN];
 #pragma unroll
         for (int t = 0; t < kLmTN; ++t) {
@@ -558,14 +559,13 @@ __global__ __launch_bounds__(256) void w8a16_large_m_kernel(const _Float16 *__re
                 acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1[t], a1, acc[t][mt], 0, 0, 0);
             }
         }
-        if (more) {
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                lds[(kt + 1) & 1][adst[i]] = areg[i];
+        for (int i = 0; i < 4; ++i)
+            lds[(kt + 1) & 1][adst[i]] = areg[i];
 #pragma unroll
-            for (int t = 0; t < kLmTN; ++t)
-                wcur[t] = wnext[t];
-        }
+        for (int t = 0; t < kLmTN; ++t)
+            wcur[t] = wnext[t];
         __syncthreads();
     }
 
@@ -639,11 +639,23 @@ static int run_gemm(const GemmArgs &a)
         }
         return EET_OK;
     }
-    const int m_blocks = (a.M + kLmBM - 1) / kLmBM, n_blocks = (a.N + kLmBN - 1) / kLmBN;
+    // 128 x 128 tiles (TN = 2) measured 5-25 % faster than 128 x 256 (TN = 4) on every prefill
+    // shape tried (M = 2048 and 8192): at ~170 registers two workgroups share a CU, and there
+    // are twice as many of them to spread over 256 CUs.  TN = 4 stays selectable for tuning.
+    const int m_blocks = (a.M + kLmBM - 1) / kLmBM;
+    bool wide = false;
+    if (const char *env = std::getenv("EET_GEMM_LARGE_M_WIDE"))  // "0" / "1": tuning override
+        wide = env[0] == '1';
+    const int bn = wide ? 256 : 128;
+    const int n_blocks = (a.N + bn - 1) / bn;
     const int total = m_blocks * n_blocks;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL(w8a16_large_m_kernel, dim3(grid), dim3(256), 0, a.st, a.A, a.Wp, a.scale, a.C, a.M, a.N, a.K,
-                       m_blocks, n_blocks, a.residual, a.epi);
+    if (wide)
+        hipLaunchKernelGGL(w8a16_large_m_kernel<4>, dim3(grid), dim3(256), 0, a.st, a.A, a.Wp, a.scale, a.C, a.M,
+                           a.N, a.K, m_blocks, n_blocks, a.residual, a.epi);
+    else
+        hipLaunchKernelGGL(w8a16_large_m_kernel<2>, dim3(grid), dim3(256), 0, a.st, a.A, a.Wp, a.scale, a.C, a.M,
+                           a.N, a.K, m_blocks, n_blocks, a.residual, a.epi);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }

@@ -153,6 +153,16 @@ __global__ __launch_bounds__(kThreads) void prefill_attention_kernel(
         __syncthreads();  // previous chunk fully consumed
         store_chunk();
         __syncthreads();
+        // ALiBi terms of this chunk's keys, requested before the prefetch below: loads return in
+        // order, so asking for them later would mean waiting for the whole next chunk as well
+        float bias[4][4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                bias[kt][r] = (alibi != nullptr) ? (float)alibi[(size_t)h * S + min(kc0 + 16 * kt + 4 * g + r, S - 1)]
+                                                 : 0.f;
+        __builtin_amdgcn_sched_barrier(0);
         if (kc0 + kBK < k_end)
             load_chunk(kc0 + kBK);
 
@@ -179,13 +189,6 @@ __global__ __launch_bounds__(kThreads) void prefill_attention_kernel(
         }
 
         // online softmax; lane (g, j) holds keys kc0 + 16*kt + 4g + r of query wq0 + 16*qt + j
-        float bias[4][4];
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                bias[kt][r] = (alibi != nullptr) ? (float)alibi[(size_t)h * S + min(kc0 + 16 * kt + 4 * g + r, S - 1)]
-                                                 : 0.f;
         half8 pop[kQT][2];
 #pragma unroll
         for (int qt = 0; qt < kQT; ++qt) {

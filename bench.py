@@ -20,7 +20,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
-LLAMA = dict(layers=32, hidden=4096, heads=32, d_ff=11008, vocab=32000)
+LLAMA = dict(layers=32, hidden=4096, heads=32, d_ff=11008, vocab=32000, alibi=False)
+BAICHUAN13B = dict(layers=40, hidden=5120, heads=40, d_ff=13696, vocab=64000, alibi=True)
 
 
 def linear_shapes(hidden, d_ff):
@@ -137,12 +138,13 @@ def cpu_baseline(torch, M, hidden, d_ff, seed, budget_s=12.0):
                       f"{per_layer * 1e3:.1f} ms per layer"}
 
 
-def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed):
-    """LLaMA-7B-shaped int8 decoder, random init: prefill `prompt` tokens then
-    greedy-decode `gen` tokens; tokens/s = batch * gen / decode time."""
+def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed, model=LLAMA):
+    """Int8 decoder of the given shape, random init: prefill `prompt` tokens then
+    greedy-decode `gen` tokens; tokens/s = batch * (gen - 1) / decode time."""
     from eet_amd import decoder as D
-    cfg = D.DecoderConfig(num_layers=len(weights), hidden=LLAMA["hidden"], heads=LLAMA["heads"], d_ff=LLAMA["d_ff"],
-                          vocab=LLAMA["vocab"], max_batch=batch, max_prompt=prompt, max_full_seq=prompt + gen + 1)
+    cfg = D.DecoderConfig(num_layers=len(weights), hidden=model["hidden"], heads=model["heads"], d_ff=model["d_ff"],
+                          vocab=model["vocab"], alibi=model["alibi"], max_batch=batch, max_prompt=prompt,
+                          max_full_seq=prompt + gen + 1)
     g = torch.Generator(device=dev).manual_seed(seed)
     H = cfg.hidden
     sd = {}
@@ -280,6 +282,9 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the M = 1..32 sweep")
+    ap.add_argument("--baichuan", action="store_true",
+                    help="also run BASELINE config 5: Baichuan-13B-shaped decoder (40 layers, ALiBi), batch 32, "
+                         "prompt 2048, 256 greedy tokens (needs ~85 GB of HBM and about a minute)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 1 GiB device-to-device copies (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -370,6 +375,15 @@ def main():
 
     if args.gen > 0:
         result["decode"] = decode_bench(torch, eet, weights, dev, args.batch, args.prompt, args.gen, seed=7)
+
+    if args.baichuan:
+        del weights, fused
+        torch.cuda.empty_cache()
+        from eet_amd import ops as _ops
+        _ops.workspaces.clear()
+        bw = make_weights(torch, eet, dev, BAICHUAN13B["layers"], BAICHUAN13B["hidden"], BAICHUAN13B["d_ff"], seed=4321)
+        result["decode_baichuan13b"] = decode_bench(torch, eet, bw, dev, 32, 2048, 256, seed=9, model=BAICHUAN13B)
+        del bw
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, M, hidden, d_ff, seed=5)

@@ -7,4 +7,7 @@ from .ops import (BaichuanMmha, CrossMultiHeadAttention, Embedding, FeedForwardN
                   pack_weights_torch, preprocess_weights, quant_weights, quant_weights_torch,
                   unpack_weights)
 
+from .convert import (convert_baichuan_weights, convert_llama_weights, convert_name,  # noqa: F401
+                      repack_reference_state_dict)
+
 __version__ = "0.1.0"

@@ -30,6 +30,7 @@ SIGNATURES = {
     "eet_qkv_split": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "eet_swiglu": (_i, [_vp, _vp, _i, _i, _vp]),
     "eet_residual_add": (_i, [_vp, _vp, _i, _i, _vp]),
+    "eet_kv_cache_reorder": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "eet_prefill_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
 }
 

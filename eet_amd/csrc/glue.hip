@@ -152,6 +152,33 @@ __global__ void residual_add_kernel(_Float16 *__restrict__ out, const _Float16 *
     reinterpret_cast<uint4 *>(out)[i] = __builtin_bit_cast(uint4, a + b);
 }
 
+// Beam-search cache reorder: dst[b] = src[index[b]] for the first `rows` time
+// steps of every head, K and V in one launch.  Replaces reorderKV
+// (csrc/core/transpose.cu:135-162), which gathers in place and says itself that
+// the read / write order is not guaranteed; here source and destination are
+// separate buffers, so the gather is exact for any index (duplicates included).
+// An index outside [0, B) copies the beam's own rows.
+// grid = (chunks, H, B); one (b, h) slab of rows*dh halves is contiguous.
+__global__ __launch_bounds__(256) void kv_reorder_kernel(const _Float16 *__restrict__ k_src,
+                                                         const _Float16 *__restrict__ v_src,
+                                                         _Float16 *__restrict__ k_dst, _Float16 *__restrict__ v_dst,
+                                                         const long long *__restrict__ index, int B, int H,
+                                                         size_t slab_stride_vec, int nvec)
+{
+    const int b = blockIdx.z, h = blockIdx.y;
+    long long from = index[b];
+    if (from < 0 || from >= B)
+        from = b;
+    const size_t so = ((size_t)from * H + h) * slab_stride_vec, dst_o = ((size_t)b * H + h) * slab_stride_vec;
+    const uint4 *ks = reinterpret_cast<const uint4 *>(k_src) + so, *vs = reinterpret_cast<const uint4 *>(v_src) + so;
+    uint4 *kd = reinterpret_cast<uint4 *>(k_dst) + dst_o, *vd = reinterpret_cast<uint4 *>(v_dst) + dst_o;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < nvec; i += gridDim.x * 256) {
+        const uint4 a = ks[i], c = vs[i];
+        kd[i] = a;
+        vd[i] = c;
+    }
+}
+
 }  // namespace
 
 extern "C" int eet_rmsnorm(const void *x, const void *gamma, void *out, int M, int N, float eps, void *stream)
@@ -223,6 +250,40 @@ extern "C" int eet_residual_add(void *out, const void *residual, int M, int N, v
     hipLaunchKernelGGL(residual_add_kernel, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<_Float16 *>(out),
                        static_cast<const _Float16 *>(residual), nvec);
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
+extern "C" int eet_kv_cache_reorder(const void *k_src, const void *v_src, void *k_dst, void *v_dst,
+                                    const int64_t *reorder_index, int B, int H, int dh, int rows, int T_cap,
+                                    void *stream)
+{
+    EET_REQUIRE(k_src && v_src && k_dst && v_dst && reorder_index, EET_ERR_INVALID_ARGUMENT,
+                "eet_kv_cache_reorder: null pointer");
+    EET_REQUIRE(B >= 0 && H > 0 && dh > 0 && rows >= 0 && rows <= T_cap, EET_ERR_INVALID_ARGUMENT,
+                "eet_kv_cache_reorder: bad sizes B=%d H=%d dh=%d rows=%d T_cap=%d", B, H, dh, rows, T_cap);
+    EET_REQUIRE(dh % 8 == 0, EET_ERR_UNSUPPORTED_SHAPE, "eet_kv_cache_reorder: head size %d must be a multiple of 8",
+                dh);
+    EET_REQUIRE(B <= 65535 && H <= 65535, EET_ERR_UNSUPPORTED_SHAPE, "eet_kv_cache_reorder: B=%d / H=%d too large", B,
+                H);
+    // The gather reads beams that other workgroups write: in place it would race.
+    const size_t bytes = (size_t)B * H * T_cap * dh * sizeof(_Float16);
+    auto overlap = [bytes](const void *a, const void *b) {
+        const char *x = static_cast<const char *>(a), *y = static_cast<const char *>(b);
+        return x < y + bytes && y < x + bytes;
+    };
+    EET_REQUIRE(!overlap(k_src, k_dst) && !overlap(v_src, v_dst) && !overlap(k_src, v_dst) && !overlap(v_src, k_dst),
+                EET_ERR_INVALID_ARGUMENT, "eet_kv_cache_reorder: source and destination caches overlap");
+    if (B == 0 || rows == 0)
+        return EET_OK;
+    const int nvec = rows * (dh / 8);
+    int chunks = (nvec + 1023) / 1024;      // >= 4 vectors per thread, all beams and heads in flight
+    if (chunks < 1)
+        chunks = 1;
+    hipLaunchKernelGGL(kv_reorder_kernel, dim3(chunks, H, B), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const _Float16 *>(k_src), static_cast<const _Float16 *>(v_src),
+                       static_cast<_Float16 *>(k_dst), static_cast<_Float16 *>(v_dst),
+                       reinterpret_cast<const long long *>(reorder_index), B, H, (size_t)T_cap * (dh / 8), nvec);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }

@@ -44,12 +44,10 @@ __device__ __forceinline__ float dot8(const u32x4 &a, const u32x4 &b)
     return s;
 }
 
-// Decode streams every cache row once (non-temporal); the prompt pass re-reads
-// rows for every query, so it keeps them cacheable.
-template <bool STREAM>
+// Decode streams every cache row exactly once: non-temporal loads.
 __device__ __forceinline__ u32x4 load_row16(const u32x4 *p)
 {
-    return STREAM ? __builtin_nontemporal_load(p) : *p;
+    return __builtin_nontemporal_load(p);
 }
 
 template <int WIDTH>
@@ -101,16 +99,13 @@ __device__ __forceinline__ u32x4 rotate8(const u32x4 &x, const u32x4 &y, int sub
 }
 
 // DH: head size.  LPR = DH/8 lanes cover one row with one 16-byte load each.
-// PREFILL = false: one query per (b, h), rows [0, step).
-// PREFILL = true : blockIdx.x also runs over the S = step prompt positions;
-//   query i of q[B][H][S][dh] attends rows [0, i] and writes ctx[b][i][h*dh..]
-//   (the causal prompt pass, one workgroup per query row; nsplit is 1).
-template <int DH, bool PREFILL, int UN>
+// One query per (b, h) attends rows [0, step); grid = (B*H, nsplit).
+template <int DH, int UN>
 __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_new, const _Float16 *__restrict__ v_new,
     long qkv_stride, _Float16 *__restrict__ k_cache, _Float16 *__restrict__ v_cache, _Float16 *__restrict__ ctx,
     const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, float *__restrict__ partial, int H,
-    int step_or_S, int T_cap, int nsplit, float scale, const float *__restrict__ rope_row)
+    int step, int T_cap, int nsplit, float scale, const float *__restrict__ rope_row)
 {
     constexpr int LPR = DH / 8;            // lanes per row
     constexpr int RPB = kThreads / LPR;    // row streams of the block (one per group of LPR lanes)
@@ -118,24 +113,19 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
     __shared__ float stream_m[RPB], stream_l[RPB];
 
     const int split = blockIdx.y;
-    const int bh = PREFILL ? blockIdx.x / step_or_S : blockIdx.x;
-    const int qi = PREFILL ? blockIdx.x % step_or_S : 0;
-    const int step = PREFILL ? qi + 1 : step_or_S;
-    const int alibi_ld = step_or_S;
+    const int bh = blockIdx.x;
+    const int alibi_ld = step;
     const int b = bh / H, h = bh % H;
     const int tid = threadIdx.x;
     const int sub = tid % LPR;   // which 8-element slice of the row
     const int rs = tid / LPR;    // which row stream
 
-    const size_t qoff = PREFILL ? (size_t)blockIdx.x * DH
-                                : (qkv_stride ? (size_t)b * qkv_stride + (size_t)h * DH : (size_t)bh * DH);
-    const size_t coff = PREFILL ? ((size_t)(b * step_or_S + qi) * H + h) * DH : (size_t)bh * DH;
+    const size_t qoff = qkv_stride ? (size_t)b * qkv_stride + (size_t)h * DH : (size_t)bh * DH;
+    const size_t coff = (size_t)bh * DH;
     _Float16 *kc = k_cache + ((size_t)b * H + h) * (size_t)T_cap * DH;
     _Float16 *vc = v_cache + ((size_t)b * H + h) * (size_t)T_cap * DH;
 
-    int t_first = pad ? (int)min((int64_t)step, max((int64_t)0, pad[b])) : 0;
-    if (PREFILL && pad && (int64_t)qi < pad[b])
-        t_first = step;  // a padded query row attends nothing and yields zeros
+    const int t_first = pad ? (int)min((int64_t)step, max((int64_t)0, pad[b])) : 0;
     const int span = step - t_first;
     const int per = (span + nsplit - 1) / nsplit;
     const int t0 = t_first + split * per;
@@ -164,7 +154,7 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
     const int r_last = own_last ? step - 1 - t0 : -1;
 
     u32x4 qv = *reinterpret_cast<const u32x4 *>(q + qoff + sub * 8);
-    if (!PREFILL && rope_row != nullptr) {
+    if (rope_row != nullptr) {
         u32x4 qy;
         qy.x = __shfl_xor(qv.x, LPR / 2, 64);
         qy.y = __shfl_xor(qv.y, LPR / 2, 64);
@@ -187,7 +177,7 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
             if (r < n)
                 kv[u] = (r == r_last)
                             ? knew
-                            : load_row16<!PREFILL>(reinterpret_cast<const u32x4 *>(kc + (size_t)(t0 + r) * DH) + sub);
+                            : load_row16(reinterpret_cast<const u32x4 *>(kc + (size_t)(t0 + r) * DH) + sub);
         }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
@@ -195,7 +185,7 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
             if (r < n)
                 vv[u] = (r == r_last)
                             ? vnew
-                            : load_row16<!PREFILL>(reinterpret_cast<const u32x4 *>(vc + (size_t)(t0 + r) * DH) + sub);
+                            : load_row16(reinterpret_cast<const u32x4 *>(vc + (size_t)(t0 + r) * DH) + sub);
         }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
@@ -300,7 +290,7 @@ int launch(const void *q, const void *k, const void *v, long qkv_stride, void *k
         const char *e = std::getenv("EET_MMHA_UNROLL");
         return e ? atoi(e) : 8;
     }();
-    auto kern = (unroll == 4) ? mmha_decode_split_kernel<DH, false, 4> : mmha_decode_split_kernel<DH, false, 8>;
+    auto kern = (unroll == 4) ? mmha_decode_split_kernel<DH, 4> : mmha_decode_split_kernel<DH, 8>;
     hipLaunchKernelGGL(kern, grid, dim3(kThreads), 0, st,
                        static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(k),
                        static_cast<const _Float16 *>(v), qkv_stride, static_cast<_Float16 *>(kc),

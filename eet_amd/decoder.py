@@ -13,7 +13,7 @@ from dataclasses import dataclass
 
 import torch
 
-from . import ops
+from . import convert, ops
 
 
 @dataclass
@@ -100,6 +100,7 @@ class Int8Decoder:
 
     def __init__(self, cfg, state_dict, device="cuda:0"):
         self.cfg = cfg
+        convert.check_layout(state_dict)
         dev = torch.device(device)
         self.desc = ops.MetaDesc(dtype=torch.float16, batch_size=cfg.max_batch, head_num=cfg.heads,
                                  hidden_units=cfg.hidden, layer_num=cfg.num_layers, max_seq_len=cfg.max_prompt,

@@ -195,6 +195,7 @@ class _MmhaInt8:
         # KV cache, private to the op (csrc/op/llama_mmha.cpp:47-48); layout [B][H][T][dh]
         self.k_cache = torch.zeros(desc.batch_size, H, self.t_cap, self.dh, dtype=torch.float16, device=dev)
         self.v_cache = torch.zeros_like(self.k_cache)
+        self._k_spare = self._v_spare = None     # second buffer of the beam-search reorder, made on first use
         self.step = 1
         self.first_batch = 0
         self.rope_table = _rope_table(self.t_cap, self.dh, dev) if self._rope else None
@@ -216,8 +217,12 @@ class _MmhaInt8:
                                f"{input.dtype} {tuple(input.shape)}")
         if input.device.type != "cuda":
             raise RuntimeError(f"[EET][ERROR] {self._name}: input must be on the GPU")
-        if reorder_state is not None and reorder_state.numel() != 0:
-            raise NotImplementedError(f"[EET][ERROR] {self._name}: beam-search cache reorder is not implemented")
+        reorder = reorder_state if (reorder_state is not None and reorder_state.numel() != 0) else None
+        if reorder is not None and not first_pass:
+            if reorder.dtype != torch.int64 or reorder.device.type != "cuda" or reorder.numel() < self.first_batch:
+                raise RuntimeError(f"[EET][ERROR] {self._name}: reorder_state must be an int64 GPU tensor with one "
+                                   f"entry per beam ({self.first_batch})")
+            reorder = reorder.contiguous()
         x = input.contiguous()
         B, S, hidden = x.shape
         if B > desc.batch_size:
@@ -248,6 +253,16 @@ class _MmhaInt8:
             t0, time_step = self.step - 1, self.step - 1
         M = B * S
         L = lib()
+        if reorder is not None and not first_pass:
+            # beam b continues from the rows of beam reorder[b] (csrc/op/llama_mmha.cpp:248-252):
+            # gather into the second cache buffer, then swap the two
+            if self._k_spare is None:
+                self._k_spare, self._v_spare = torch.zeros_like(self.k_cache), torch.zeros_like(self.v_cache)
+            check(L.eet_kv_cache_reorder(self.k_cache.data_ptr(), self.v_cache.data_ptr(), self._k_spare.data_ptr(),
+                                         self._v_spare.data_ptr(), reorder.data_ptr(), self.first_batch, H, dh,
+                                         self.step - 1, self.t_cap, _stream()), "eet_kv_cache_reorder")
+            self.k_cache, self._k_spare = self._k_spare, self.k_cache
+            self.v_cache, self._v_spare = self._v_spare, self.v_cache
         f16 = torch.float16
         xn = workspaces.get("layernorm", desc.batch_size * max(desc.max_seq_len, 1) * hidden, f16, dev)
         qkv = workspaces.get("qkv", desc.batch_size * max(desc.max_seq_len, 1) * 3 * self.inner, f16, dev)
@@ -294,7 +309,7 @@ class _MmhaInt8:
                   "eet_mmha_decode")
         # output projection with the residual add (csrc/op/llama_mmha.cpp:428-462) in its epilogue
         _gemm(cbuf, self.o_w, self.o_s, out, M, hidden, self.inner, EPI_RESIDUAL, x)
-        self._keep = (x, pad, alibi)  # inputs of kernels still in flight
+        self._keep = (x, pad, alibi, reorder)  # inputs of kernels still in flight
         return out[: M * hidden].view(B, S, hidden)
 
 

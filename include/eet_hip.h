@@ -168,6 +168,17 @@ int eet_swiglu(void *gate, const void *up, int M, int N, void *stream);
  * bias == nullptr (csrc/core/add_bias.cu:51-73). */
 int eet_residual_add(void *out, const void *residual, int M, int N, void *stream);
 
+/* Beam-search cache reorder: dst[b][h][t][:] = src[reorder_index[b]][h][t][:]
+ * for t < rows, K and V, caches [B][H][T_cap][dh] half, reorder_index int64[B]
+ * in device memory (an entry outside [0, B) keeps the beam's own rows).  src
+ * and dst must not overlap: the caller keeps two cache buffers and swaps them.
+ * Replaces reorderKV_kernel (csrc/core/transpose.cu:135-162) as called from
+ * LlamaMmha::reorder_cache (csrc/op/llama_mmha.cpp:248-252, 495-508), whose
+ * in-place form does not order its reads before its writes. */
+int eet_kv_cache_reorder(const void *k_src, const void *v_src, void *k_dst, void *v_dst,
+                         const int64_t *reorder_index, int B, int H, int dh, int rows, int T_cap,
+                         void *stream);
+
 /* Causal prefill attention over the prompt, reading K and V from the caches
  * filled by eet_qkv_split.  q [B][H][S][dh]; ctx [B][S][H*dh]; alibi NULL or
  * [H][S] half (slope * j, the diagonal row of the reference's mask); pad as in

@@ -210,6 +210,17 @@ def alibi_mask(n_head, length):
 # ----------------------------------------------------------------------------
 # layer / decoder composition
 # ----------------------------------------------------------------------------
+def reorder_cache(k_cache, v_cache, index, rows):
+    """Beam-search gather: beam b takes over the first `rows` time steps of beam
+    index[b].  csrc/core/transpose.cu:135-152 (reorderKV) as called from
+    csrc/op/llama_mmha.cpp:248-252; the gather is taken from a snapshot, which is
+    what that in-place kernel means to compute.  Caches [B][H][T][dh]."""
+    ks, vs = k_cache.copy(), v_cache.copy()
+    for b, src in enumerate(index):
+        k_cache[b, :, :rows] = ks[src, :, :rows]
+        v_cache[b, :, :rows] = vs[src, :, :rows]
+
+
 class OracleAttention:
     """LlamaMmha / BaichuanMmha restated.  csrc/op/llama_mmha.cpp:114-266,
     csrc/op/baichuan_mmha.cpp:81-216.  Weights are the *unprocessed* int8
@@ -222,9 +233,11 @@ class OracleAttention:
         self.v_cache = np.zeros((B, H, cap, dh), F16)
         self.step = 1
 
-    def forward(self, x, pad, first_pass, alibi=None):
+    def forward(self, x, pad, first_pass, alibi=None, reorder=None):
         B, S, hidden = x.shape
         H, dh = self.H, self.dh
+        if reorder is not None and not first_pass:
+            reorder_cache(self.k_cache, self.v_cache, reorder, self.step)
         xn = rmsnorm(x.reshape(B * S, hidden), self.gamma, self.eps)
         qkv = dequant_matmul(xn, self.qkv_q, self.qkv_s)
         if first_pass:

@@ -86,3 +86,49 @@ def test_prefill_attention(gpu, B, H, S, dh, use_pad, use_alibi):
                                       ctx.data_ptr(), row.data_ptr() if use_alibi else None,
                                       padd.data_ptr() if use_pad else None, B, H, S, dh, cap, stream()))
     assert_close(ctx.cpu().numpy(), want, what="prefill ctx")
+
+
+@pytest.mark.parametrize("B,H,dh,rows,cap", [(4, 3, 64, 9, 16), (8, 32, 128, 100, 128), (3, 2, 32, 0, 8),
+                                             (5, 4, 128, 40, 40)])
+def test_kv_cache_reorder(gpu, B, H, dh, rows, cap):
+    """Gather with repeated sources; rows at and after `rows` of the destination stay as they were.
+    Bit-exact against the oracle's snapshot gather."""
+    g = torch.Generator().manual_seed(B * 100 + rows)
+    k = torch.randn(B, H, cap, dh, generator=g).half()
+    v = torch.randn(B, H, cap, dh, generator=g).half()
+    idx = torch.randint(0, B, (B,), generator=g)
+    idx[0] = idx[-1] = B - 1                      # a source used twice, and beam 0 overwritten
+    kd0 = torch.randn(B, H, cap, dh, generator=g).half()
+    vd0 = torch.randn(B, H, cap, dh, generator=g).half()
+    dk, dv, dkd, dvd, didx = k.to(gpu), v.to(gpu), kd0.to(gpu), vd0.to(gpu), idx.to(gpu)
+    check(lib().eet_kv_cache_reorder(dk.data_ptr(), dv.data_ptr(), dkd.data_ptr(), dvd.data_ptr(), didx.data_ptr(),
+                                     B, H, dh, rows, cap, stream()), "eet_kv_cache_reorder")
+    torch.cuda.synchronize()
+    wk, wv = k.numpy().copy(), v.numpy().copy()
+    O.reorder_cache(wk, wv, idx.numpy(), rows)
+    wk[:, :, rows:], wv[:, :, rows:] = kd0.numpy()[:, :, rows:], vd0.numpy()[:, :, rows:]
+    assert np.array_equal(dkd.cpu().numpy().view(np.uint16), wk.view(np.uint16))
+    assert np.array_equal(dvd.cpu().numpy().view(np.uint16), wv.view(np.uint16))
+    # the sources are untouched
+    assert torch.equal(dk.cpu(), k) and torch.equal(dv.cpu(), v)
+
+
+def test_kv_cache_reorder_arguments(gpu):
+    B, H, dh, cap = 2, 2, 64, 8
+    k = torch.zeros(B, H, cap, dh, dtype=torch.float16, device=gpu)
+    v, k2, v2 = torch.zeros_like(k), torch.zeros_like(k), torch.zeros_like(k)
+    idx = torch.tensor([5, -1], device=gpu)          # out of range: the beam keeps its own rows
+    k.copy_(torch.arange(k.numel(), device=gpu).view_as(k) % 97)
+    L = lib()
+    assert L.eet_kv_cache_reorder(k.data_ptr(), v.data_ptr(), k2.data_ptr(), v2.data_ptr(), idx.data_ptr(), B, H, dh,
+                                  4, cap, stream()) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(k2[:, :, :4], k[:, :, :4]) and not k2[:, :, 4:].any()
+    # in place would race: refused
+    assert L.eet_kv_cache_reorder(k.data_ptr(), v.data_ptr(), k.data_ptr(), v2.data_ptr(), idx.data_ptr(), B, H, dh,
+                                  4, cap, stream()) == -1
+    assert b"overlap" in L.eet_last_error()
+    assert L.eet_kv_cache_reorder(k.data_ptr(), v.data_ptr(), k2.data_ptr(), v2.data_ptr(), idx.data_ptr(), B, H, dh,
+                                  9, cap, stream()) == -1
+    assert L.eet_kv_cache_reorder(k.data_ptr(), v.data_ptr(), k2.data_ptr(), v2.data_ptr(), idx.data_ptr(), B, H, 12,
+                                  4, cap, stream()) == -2

@@ -144,3 +144,82 @@ def test_greedy_tokens_match_oracle(gpu, alibi):
     model2 = D.Int8Decoder(cfg, sd, device="cuda:0")
     toks = model2.greedy(ids.to(gpu), 4).cpu().numpy()
     assert toks.shape == (3, 4)
+
+
+def test_converted_checkpoint_runs(gpu):
+    """HF-named fp16 LLaMA weights -> convert_llama_weights -> Int8Decoder, against an oracle
+    decoder whose int8 weights come from the oracle's own quantiser on the same fp16 matrices."""
+    from eet_amd import convert
+    from oracle import quant as oq
+    cfg = tiny_cfg(False)
+    g = torch.Generator().manual_seed(11)
+    r = lambda *s: (torch.randn(*s, generator=g) * 0.02).half()
+    H, F = cfg.hidden, cfg.d_ff
+    hf = {"model.embed_tokens.weight": r(cfg.vocab, H), "model.norm.weight": 1 + 5 * r(H),
+          "lm_head.weight": 8 * r(cfg.vocab, H)}
+    for i in range(cfg.num_layers):
+        p = f"model.layers.{i}."
+        for n in "qkvo":
+            hf[p + f"self_attn.{n}_proj.weight"] = r(H, H)
+        hf[p + "mlp.gate_proj.weight"], hf[p + "mlp.up_proj.weight"] = r(F, H), r(F, H)
+        hf[p + "mlp.down_proj.weight"] = r(H, F)
+        hf[p + "input_layernorm.weight"], hf[p + "post_attention_layernorm.weight"] = 1 + 5 * r(H), 1 + 5 * r(H)
+    sd = convert.convert_llama_weights(hf, torch.int8)
+    model = D.Int8Decoder(cfg, sd, device="cuda:0")
+
+    def oq_lin(w_hf):
+        q, s = oq.quantize_ref128(w_hf.t().contiguous().numpy())
+        return torch.from_numpy(q), torch.from_numpy(s)
+    raw = {}
+    for i in range(cfg.num_layers):
+        p, pre = f"model.layers.{i}.", f"layer.{i}."
+        raw[pre + "self_attn.qkv_proj"] = oq_lin(torch.cat([hf[p + f"self_attn.{n}_proj.weight"] for n in "qkv"], 0))
+        raw[pre + "self_attn.out_proj"] = oq_lin(hf[p + "self_attn.o_proj.weight"])
+        raw[pre + "ffn.intermediate_0"] = oq_lin(hf[p + "mlp.gate_proj.weight"])
+        raw[pre + "ffn.intermediate_1"] = oq_lin(hf[p + "mlp.up_proj.weight"])
+        raw[pre + "ffn.output"] = oq_lin(hf[p + "mlp.down_proj.weight"])
+    ref = oracle_decoder(cfg, sd, raw)
+    ids = torch.randint(0, cfg.vocab, (2, 7), generator=g)
+    logits = ref.step(ids.numpy(), True)
+    got = model.logits(ids.to(gpu), True).float().cpu().numpy()[:, 0]
+    assert_close(got, logits, 3e-2, 3e-2, "prefill logits")
+    nxt = logits.argmax(-1)
+    logits = ref.step(nxt[:, None], False)
+    got = model.logits(torch.from_numpy(nxt)[:, None].to(gpu), False).float().cpu().numpy()[:, 0]
+    assert_close(got, logits, 3e-2, 3e-2, "decode logits")
+
+    # a dict carrying the reference's layout tag is refused rather than mis-read
+    bad = dict(sd)
+    bad[convert.LAYOUT_KEY] = convert.LAYOUT_REF_SM80
+    with pytest.raises(RuntimeError, match="layout"):
+        D.Int8Decoder(cfg, bad, device="cuda:0")
+
+
+@pytest.mark.parametrize("alibi", [False, True])
+def test_beam_search_reorder(gpu, alibi):
+    """reorder_state on incremental calls: beam b continues from the cache rows of beam
+    reorder_state[b] (llama_mmha.cpp:248-252), including a beam that is dropped and one taken twice."""
+    cfg = tiny_cfg(alibi, layers=1)
+    sd, raw = D.random_state_dict(cfg, seed=9)
+    attn = D.Int8Decoder(cfg, sd, device="cuda:0").layers[0][0]
+    oattn = oracle_decoder(cfg, sd, raw).layers[0][0]
+    g = torch.Generator().manual_seed(4)
+    B, S = 3, 5
+    e = torch.empty(0, dtype=torch.long)
+    x = torch.randn(B, S, cfg.hidden, generator=g).half()
+    attn.forward(x.to(gpu), e, e, True, True, True, D.alibi_mask(cfg.heads, S).to(gpu) if alibi else torch.empty(0))
+    oattn.forward(x.numpy(), None, True, O.alibi_mask(cfg.heads, S) if alibi else None)
+    orders = [None, [2, 0, 0], [1, 1, 2], None, [0, 2, 1]]
+    for t, order in enumerate(orders):
+        step = S + t + 1
+        x1 = torch.randn(B, 1, cfg.hidden, generator=g).half()
+        bias = D.alibi_mask(cfg.heads, step)[:, -1:, :].contiguous().to(gpu) if alibi else torch.empty(0)
+        ro = torch.tensor(order, dtype=torch.long, device=gpu) if order is not None else e
+        y = attn.forward(x1.to(gpu), e, ro, True, True, False, bias)
+        want = oattn.forward(x1.numpy(), None, False, O.alibi_bias(cfg.heads, step) if alibi else None, reorder=order)
+        assert_close(y.cpu().numpy(), want, RT, AT, f"attention step {t} order {order}")
+    assert_close(attn.k_cache[:, :, :step].cpu().numpy(), oattn.k_cache[:, :, :step], 4e-3, 4e-3, "k cache")
+    assert_close(attn.v_cache[:, :, :step].cpu().numpy(), oattn.v_cache[:, :, :step], 4e-3, 4e-3, "v cache")
+    with pytest.raises(RuntimeError, match="reorder_state"):
+        attn.forward(x1.to(gpu), e, torch.tensor([0, 1, 2], dtype=torch.int32, device=gpu), True, True, False,
+                     D.alibi_mask(cfg.heads, step + 1)[:, -1:, :].contiguous().to(gpu) if alibi else torch.empty(0))

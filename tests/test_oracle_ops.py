@@ -188,3 +188,25 @@ def test_cpu_path_matches_numpy_oracle():
     got = cpu_path.dequant_matmul(torch.from_numpy(x), torch.from_numpy(q), torch.from_numpy(s)).numpy()
     want = O.dequant_matmul(x, q, s)
     assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=2e-3, atol=1e-4)
+
+
+def test_reorder_cache_gather():
+    """reorder_cache: element-by-element definition (brute force), a permutation undone by its
+    inverse, and a repeated source -- an in-place loop over beams would fail the last two."""
+    rng = np.random.default_rng(8)
+    B, H, T, dh, rows = 4, 2, 6, 8, 4
+    k0 = rng.standard_normal((B, H, T, dh)).astype(np.float16)
+    v0 = rng.standard_normal((B, H, T, dh)).astype(np.float16)
+    idx = [1, 0, 0, 2]                       # 0 <-> 1 swap (in-place order trap) + a source used twice
+    k, v = k0.copy(), v0.copy()
+    O.reorder_cache(k, v, idx, rows)
+    for b in range(B):
+        for h in range(H):
+            for t in range(T):
+                src = idx[b] if t < rows else b
+                assert np.array_equal(k[b, h, t], k0[src, h, t]) and np.array_equal(v[b, h, t], v0[src, h, t])
+    perm, inv = [2, 3, 1, 0], [3, 2, 0, 1]
+    k, v = k0.copy(), v0.copy()
+    O.reorder_cache(k, v, perm, T)
+    O.reorder_cache(k, v, inv, T)
+    assert np.array_equal(k, k0) and np.array_equal(v, v0)

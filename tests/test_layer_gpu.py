@@ -107,9 +107,9 @@ def test_op_validation(gpu):
         attn.forward(torch.zeros(1, 1, cfg.hidden, dtype=torch.float16, device=gpu), e, e, True, True, False)
     with pytest.raises(RuntimeError, match="seq_len 1"):
         attn.forward(torch.zeros(1, 2, cfg.hidden, dtype=torch.float16, device=gpu), e, e, True, True, False)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError, match="reorder_state"):
         attn.forward(torch.zeros(1, 1, cfg.hidden, dtype=torch.float16, device=gpu), e,
-                     torch.zeros(1, dtype=torch.long, device=gpu), True, True, False)
+                     torch.zeros(1, dtype=torch.long), True, True, False)          # CPU tensor
     with pytest.raises(RuntimeError, match="fp16"):
         ffn.forward(torch.zeros(1, 1, cfg.hidden, device=gpu), True, True)
 

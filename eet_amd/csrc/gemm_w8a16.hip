@@ -27,38 +27,11 @@
 
 #include <cstdlib>
 
-#include "common.h"
+#include "gemm_common.h"
+
+using namespace eet;
 
 namespace {
-
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-// 4 biased bytes -> 4 fp16 values (q = u8 - 128), exact.
-__device__ __forceinline__ void widen4(uint32_t x, half2v &lo, half2v &hi)
-{
-    const half2v magic = {(_Float16)1152.0f, (_Float16)1152.0f};
-    uint32_t a = __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u);  // {0x64, b1, 0x64, b0}
-    uint32_t b = __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);  // {0x64, b3, 0x64, b2}
-    lo = __builtin_bit_cast(half2v, a) - magic;
-    hi = __builtin_bit_cast(half2v, b) - magic;
-}
-
-__device__ __forceinline__ half8 widen8(uint32_t x0, uint32_t x1)
-{
-    half2v a, b, c, d;
-    widen4(x0, a, b);
-    widen4(x1, c, d);
-    half8 r = {a.x, a.y, b.x, b.y, c.x, c.y, d.x, d.y};
-    return r;
-}
-
-// Epilogues: plain; + residual[M][N] (fp16 add); SwiGLU over (gate, up) n-tile
-// pairs of an interleaved weight, output [M][N/2].
-constexpr int kEpiNone = 0, kEpiResidual = 1, kEpiSwiglu = 2;
 
 // One batch of U k-tiles as it comes back from memory: the raw weight tiles of
 // NT n-tiles, and the activations of RG groups of 8 rows, loaded row-wise.
@@ -355,19 +328,6 @@ struct SmallMConfig {
     int nt, waves, u;
 };
 
-struct GemmArgs {
-    const _Float16 *A;
-    const u32x4 *Wp;
-    const _Float16 *scale;
-    _Float16 *C;
-    int M, N, K;
-    const _Float16 *residual;
-    int epi;
-    const _Float16 *rms_gamma;  // non-null: RMSnorm prologue (small-M kernel only)
-    float rms_eps;
-    hipStream_t st;
-};
-
 template <int NT, int RG, int WAVES, int U, bool RMS>
 int launch_small_m(const GemmArgs &a)
 {
@@ -455,168 +415,6 @@ int run_small_m(const GemmArgs &a)
     return dispatch_small_m<4>(cfg, a);
 }
 
-// ---------------------------------------------------------------------------
-// Large-M kernel (M > 32, prefill; fp16-MFMA bound).
-//
-// Block tile 128 (M) x 256 or 128 (N) x 64 (K), 4 wavefronts side by side along N,
-// each 8 m-tiles x TN (4 or 2) n-tiles of v_mfma_f32_16x16x32_f16 (128 or 64 fp32
-// accumulator registers).  Weights: every wavefront reads its own four packed
-// tiles straight from global memory into registers -- the packed layout is
-// already the MFMA operand layout, so they never touch LDS -- and widens them
-// once per k-tile.  Activations: the block's 128 x 64 slab is loaded row-wise
-// (whole 128-byte lines), written to LDS in operand order with an XOR swizzle
-// (conflict-free 16-byte writes and reads) and read by all four wavefronts.
-// Both streams are prefetched one k-tile ahead; one barrier per k-tile.
-// Workgroups are numbered so that the ones sharing a weight column block run
-// on the same XCD (workgroup i lands on XCD i % 8) and hit its L2.
-// ---------------------------------------------------------------------------
-constexpr int kLmBM = 128, kLmTM = kLmBM / 16;  // the block is 128 rows x (4 wavefronts x TN n-tiles x 16) channels
-
-template <int kLmTN>
-__global__ __launch_bounds__(256) void w8a16_large_m_kernel(const _Float16 *__restrict__ A,
-                                                            const u32x4 *__restrict__ Wp,
-                                                            const _Float16 *__restrict__ scale,
-                                                            _Float16 *__restrict__ C, int M, int N, int K,
-                                                            int m_blocks, int n_blocks,
-                                                            const _Float16 *__restrict__ residual, int epi)
-{
-    __shared__ u32x4 lds[2][kLmTM * 2 * 64];  // [buffer][(mt*2+h)*64 + slot], 16 KiB each
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int g = lane >> 4, j = lane & 15;
-    const int ktiles = K >> 6, ntiles = N >> 4;
-
-    // XCD-aware tile order: consecutive workgroups of one XCD walk down the
-    // m-blocks of the same n-block.
-    const int total = m_blocks * n_blocks;
-    const int per_xcd = (total + 7) / 8;
-    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (tile >= total)
-        return;
-    const int n_blk = tile / m_blocks, m_blk = tile % m_blocks;
-    const int m0 = m_blk * kLmBM;
-    const int nt0 = n_blk * (4 * kLmTN) + wave * kLmTN;
-
-    const u32x4 *wbase[kLmTN];
-#pragma unroll
-    for (int t = 0; t < kLmTN; ++t)
-        wbase[t] = Wp + (size_t)min(nt0 + t, ntiles - 1) * ktiles * 64 + lane;
-
-    // activation pieces: 128 rows x 8 pieces of 16 bytes = 1024, four per thread
-    const u32x4 *asrc[4];
-    int adst[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int q = tid + 256 * i, row = q >> 3, p = q & 7;
-        asrc[i] = reinterpret_cast<const u32x4 *>(A + (size_t)min(m0 + row, M - 1) * K) + p;
-        adst[i] = ((row >> 4) * 2 + (p & 1)) * 64 + (p >> 1) * 16 + ((row & 15) ^ p);
-    }
-
-    floatx4 acc[kLmTN][kLmTM];
-#pragma unroll
-    for (int t = 0; t < kLmTN; ++t)
-#pragma unroll
-        for (int mt = 0; mt < kLmTM; ++mt)
-            acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    u32x4 wcur[kLmTN], wnext[kLmTN], areg[4];
-#pragma unroll
-    for (int t = 0; t < kLmTN; ++t)
-        wcur[t] = wbase[t][0];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        areg[i] = asrc[i][0];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        lds[0][adst[i]] = areg[i];
-    __syncthreads();
-
-    const int rslot0 = g * 16 + (j ^ (2 * g)), rslot1 = g * 16 + (j ^ (2 * g + 1));
-    for (int kt = 0; kt < ktiles; ++kt) {
-        // prefetch the next k-tile (the last iteration re-reads its own tile: no branch around the loads)
-        const int kn = min(kt + 1, ktiles - 1);
-#pragma unroll
-        for (int t = 0; t < kLmTN; ++t)
-            wnext[t] = wbase[t][(size_t)kn * 64];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            areg[i] = asrc[i][kn * 8];
-        __builtin_amdgcn_sched_barrier(0);
-        half8 w0[kLmTN], w1[kLmTN];
-#pragma unroll
-        for (int t = 0; t < kLmTN; ++t) {
-            w0[t] = widen8(wcur[t].x, wcur[t].y);
-            w1[t] = widen8(wcur[t].z, wcur[t].w);
-        }
-        const u32x4 *buf = lds[kt & 1];
-#pragma unroll
-        for (int mt = 0; mt < kLmTM; ++mt) {
-            const half8 a0 = __builtin_bit_cast(half8, buf[(mt * 2) * 64 + rslot0]);
-            const half8 a1 = __builtin_bit_cast(half8, buf[(mt * 2 + 1) * 64 + rslot1]);
-#pragma unroll
-            for (int t = 0; t < kLmTN; ++t) {
-                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0[t], a0, acc[t][mt], 0, 0, 0);
-                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1[t], a1, acc[t][mt], 0, 0, 0);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            lds[(kt + 1) & 1][adst[i]] = areg[i];
-#pragma unroll
-        for (int t = 0; t < kLmTN; ++t)
-            wcur[t] = wnext[t];
-        __syncthreads();
-    }
-
-    // acc[t][mt][r] of lane (g, j): row m0 + 16*mt + j, channel 16*(nt0+t) + 4*g + r
-    if (epi == kEpiSwiglu) {
-#pragma unroll
-        for (int t = 0; t < kLmTN; t += 2) {
-            if (nt0 + t + 1 >= ntiles)
-                continue;
-            const half4 sg = *reinterpret_cast<const half4 *>(scale + (nt0 + t) * 16 + 4 * g);
-            const half4 su = *reinterpret_cast<const half4 *>(scale + (nt0 + t + 1) * 16 + 4 * g);
-            const int n = ((nt0 + t) / 2) * 16 + 4 * g;
-#pragma unroll
-            for (int mt = 0; mt < kLmTM; ++mt) {
-                const int m = m0 + 16 * mt + j;
-                if (m < M) {
-                    half4 o;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float gate = (float)(_Float16)(acc[t][mt][r] * (float)sg[r]);
-                        const float up = (float)(_Float16)(acc[t + 1][mt][r] * (float)su[r]);
-                        o[r] = (_Float16)(up * gate / (1.0f + __expf(-gate)));
-                    }
-                    *reinterpret_cast<half4 *>(C + (size_t)m * (N / 2) + n) = o;
-                }
-            }
-        }
-        return;
-    }
-#pragma unroll
-    for (int t = 0; t < kLmTN; ++t) {
-        if (nt0 + t >= ntiles)
-            continue;
-        const int n = (nt0 + t) * 16 + 4 * g;
-        const half4 sc = *reinterpret_cast<const half4 *>(scale + n);
-#pragma unroll
-        for (int mt = 0; mt < kLmTM; ++mt) {
-            const int m = m0 + 16 * mt + j;
-            if (m < M) {
-                half4 o;
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    o[r] = (_Float16)(acc[t][mt][r] * (float)sc[r]);
-                if (epi == kEpiResidual)
-                    o = o + *reinterpret_cast<const half4 *>(residual + (size_t)m * N + n);
-                *reinterpret_cast<half4 *>(C + (size_t)m * N + n) = o;
-            }
-        }
-    }
-}
-
 }  // namespace
 
 static int run_gemm(const GemmArgs &a)
@@ -639,25 +437,7 @@ static int run_gemm(const GemmArgs &a)
         }
         return EET_OK;
     }
-    // 128 x 128 tiles (TN = 2) measured 5-25 % faster than 128 x 256 (TN = 4) on every prefill
-    // shape tried (M = 2048 and 8192): at ~170 registers two workgroups share a CU, and there
-    // are twice as many of them to spread over 256 CUs.  TN = 4 stays selectable for tuning.
-    const int m_blocks = (a.M + kLmBM - 1) / kLmBM;
-    bool wide = false;
-    if (const char *env = std::getenv("EET_GEMM_LARGE_M_WIDE"))  // "0" / "1": tuning override
-        wide = env[0] == '1';
-    const int bn = wide ? 256 : 128;
-    const int n_blocks = (a.N + bn - 1) / bn;
-    const int total = m_blocks * n_blocks;
-    const int grid = ((total + 7) / 8) * 8;
-    if (wide)
-        hipLaunchKernelGGL(w8a16_large_m_kernel<4>, dim3(grid), dim3(256), 0, a.st, a.A, a.Wp, a.scale, a.C, a.M,
-                           a.N, a.K, m_blocks, n_blocks, a.residual, a.epi);
-    else
-        hipLaunchKernelGGL(w8a16_large_m_kernel<2>, dim3(grid), dim3(256), 0, a.st, a.A, a.Wp, a.scale, a.C, a.M,
-                           a.N, a.K, m_blocks, n_blocks, a.residual, a.epi);
-    EET_HIP_CHECK(hipGetLastError());
-    return EET_OK;
+    return eet::run_large_m(a);
 }
 
 static int check_gemm_args(const char *fn, const void *A, const void *W, const void *scale, const void *C, int M,

@@ -1,0 +1,519 @@
+// Large-M fused dequant-GEMM (M > 128, prefill; fp16-MFMA bound).
+//
+// Replaces the tensor-core side of fastertransformer::gemm_fp16_int_bias_act<uint8_t>
+// (3rdparty/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm_template.h:48-177).
+//
+// A workgroup of WMW x WNW wavefronts owns a block tile of (WMW*TM*16) rows x
+// (WNW*TN*16) channels; each wavefront owns TM x TN tiles of
+// v_mfma_f32_16x16x32_f16 (TM*TN*4 fp32 accumulator registers).  What bounds
+// such a kernel on a CU is the LDS port (128 B/clk) against the matrix cores
+// (4 x 1024 flop/clk): a wavefront tile of WM x WN outputs needs (WM + WN) * 2 B
+// of operands per k for 2 * WM * WN flop, so wavefront tiles are made large
+// (128 x 64) and only one operand goes through LDS:
+//   weights      every wavefront reads its own TN packed tiles straight from
+//                global memory into registers -- the packed layout is already
+//                the MFMA operand layout -- and widens them once per k-tile;
+//   activations  the block's rows x 64 slab is loaded row-wise (whole 128-byte
+//                lines), written to LDS in operand order with an XOR swizzle
+//                (conflict-free 16-byte writes and reads) and read by every
+//                wavefront of its row group.
+// Both streams are prefetched one k-tile ahead into registers; LDS is double
+// buffered, one barrier per k-tile.  Workgroups are numbered so that the ones
+// sharing a weight column block run on the same XCD (workgroup i lands on XCD
+// i % 8) and hit its L2.
+#include <cstdlib>
+
+#include "gemm_common.h"
+
+using namespace eet;
+
+namespace {
+
+template <int WMW, int WNW, int TM, int TN>
+struct LmShape {
+    static constexpr int kThreads = 64 * WMW * WNW;
+    static constexpr int kBM = WMW * TM * 16, kBN = WNW * TN * 16;
+    static constexpr int kPieces = kBM * 8 / kThreads;  // 16-byte activation pieces per thread and k-tile
+    static constexpr int kBufVec = (kBM / 16) * 2 * 64; // u32x4 per LDS buffer: [m-tile][k-half][64 slots]
+    static_assert(kBM * 8 % kThreads == 0, "activation slab must divide evenly over the threads");
+    static_assert(2 * kBufVec * 16 <= 65536, "two activation buffers must fit 64 KiB");
+};
+
+template <int WMW, int WNW, int TM, int TN>
+__global__ __launch_bounds__(64 * WMW * WNW) __attribute__((amdgpu_waves_per_eu(2))) void w8a16_large_m_kernel(
+    const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
+    _Float16 *__restrict__ C, int M, int N, int K, int m_blocks, int n_blocks,
+    const _Float16 *__restrict__ residual, int epi)
+{
+    using S = LmShape<WMW, WNW, TM, TN>;
+    __shared__ u32x4 lds[2][S::kBufVec];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WNW, wn = wave % WNW;
+    const int g = lane >> 4, j = lane & 15;
+    const int ktiles = K >> 6, ntiles = N >> 4;
+
+    // XCD-aware tile order: consecutive workgroups of one XCD walk down the
+    // m-blocks of the same n-block.
+    const int total = m_blocks * n_blocks;
+    const int per_xcd = (total + 7) / 8;
+    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (tile >= total)
+        return;
+    const int n_blk = tile / m_blocks, m_blk = tile % m_blocks;
+    const int m0 = m_blk * S::kBM;
+    const int nt0 = n_blk * (WNW * TN) + wn * TN;
+
+    // A tile index past the end is clamped: its results are never written.
+    const u32x4 *wbase[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+        wbase[t] = Wp + (size_t)min(nt0 + t, ntiles - 1) * ktiles * 64 + lane;
+
+    // Activation pieces: rows x 8 pieces of 16 bytes.  Piece p of row r goes to
+    // block (r/16, p%2), slot (p/2)*16 + ((r%16) ^ p): lane (g, j) of k-half h
+    // then finds its operand (piece 2g+h of row j) at slot g*16 + (j ^ (2g+h)).
+    // Rows past M read row M-1; those outputs are never written.
+    const u32x4 *asrc[S::kPieces];
+    int adst[S::kPieces];
+#pragma unroll
+    for (int i = 0; i < S::kPieces; ++i) {
+        const int q = tid + S::kThreads * i, row = q >> 3, p = q & 7;
+        asrc[i] = reinterpret_cast<const u32x4 *>(A + (size_t)min(m0 + row, M - 1) * K) + p;
+        adst[i] = ((row >> 4) * 2 + (p & 1)) * 64 + (p >> 1) * 16 + ((row & 15) ^ p);
+    }
+
+    floatx4 acc[TN][TM];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt)
+            acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    u32x4 wcur[TN], wnext[TN], areg[S::kPieces];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+        wcur[t] = wbase[t][0];
+#pragma unroll
+    for (int i = 0; i < S::kPieces; ++i)
+        areg[i] = asrc[i][0];
+#pragma unroll
+    for (int i = 0; i < S::kPieces; ++i)
+        lds[0][adst[i]] = areg[i];
+    __syncthreads();
+
+    const int rslot0 = wm * TM * 128 + g * 16 + (j ^ (2 * g)), rslot1 = wm * TM * 128 + 64 + g * 16 + (j ^ (2 * g + 1));
+    for (int kt = 0; kt < ktiles; ++kt) {
+        // prefetch the next k-tile (the last iteration re-reads its own tile: no branch around the loads)
+        const int kn = min(kt + 1, ktiles - 1);
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+            wnext[t] = wbase[t][(size_t)kn * 64];
+#pragma unroll
+        for (int i = 0; i < S::kPieces; ++i)
+            areg[i] = asrc[i][kn * 8];
+        __builtin_amdgcn_sched_barrier(0);
+        half8 w0[TN], w1[TN];
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+            w0[t] = widen8(wcur[t].x, wcur[t].y);
+            w1[t] = widen8(wcur[t].z, wcur[t].w);
+        }
+        const u32x4 *buf = lds[kt & 1];
+        // The A operands of m-tile mt+1 are requested before the products of m-tile
+        // mt are issued, into the other register pair (the group barriers below pin
+        // that order; left alone the scheduler reuses one pair and waits on every read).
+        half8 aop[2][2];
+        aop[0][0] = __builtin_bit_cast(half8, buf[rslot0]);
+        aop[0][1] = __builtin_bit_cast(half8, buf[rslot1]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt) {
+            if (mt + 1 < TM) {
+                aop[(mt + 1) & 1][0] = __builtin_bit_cast(half8, buf[(mt + 1) * 128 + rslot0]);
+                aop[(mt + 1) & 1][1] = __builtin_bit_cast(half8, buf[(mt + 1) * 128 + rslot1]);
+            }
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0[t], aop[mt & 1][0], acc[t][mt], 0, 0, 0);
+                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1[t], aop[mt & 1][1], acc[t][mt], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt) {
+            if (mt + 1 < TM)
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // 2 LDS reads
+            __builtin_amdgcn_sched_group_barrier(0x008, 2 * TN, 0);  // 2*TN MFMA
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < S::kPieces; ++i)
+            lds[(kt + 1) & 1][adst[i]] = areg[i];
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+            wcur[t] = wnext[t];
+        __syncthreads();
+    }
+
+    // acc[t][mt][r] of lane (g, j): row m0 + 16*(wm*TM + mt) + j, channel 16*(nt0+t) + 4*g + r
+    const int mrow0 = m0 + 16 * wm * TM + j;
+    if (epi == kEpiSwiglu) {
+        if constexpr (TN % 2 == 0) {
+#pragma unroll
+            for (int t = 0; t < TN; t += 2) {
+                if (nt0 + t + 1 >= ntiles)
+                    continue;
+                const half4 sg = *reinterpret_cast<const half4 *>(scale + (nt0 + t) * 16 + 4 * g);
+                const half4 su = *reinterpret_cast<const half4 *>(scale + (nt0 + t + 1) * 16 + 4 * g);
+                const int n = ((nt0 + t) / 2) * 16 + 4 * g;
+#pragma unroll
+                for (int mt = 0; mt < TM; ++mt) {
+                    const int m = mrow0 + 16 * mt;
+                    if (m < M) {
+                        half4 o;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            // gate and up are rounded to fp16 first, as the separate GEMMs would leave them
+                            const float gate = (float)(_Float16)(acc[t][mt][r] * (float)sg[r]);
+                            const float up = (float)(_Float16)(acc[t + 1][mt][r] * (float)su[r]);
+                            o[r] = (_Float16)(up * gate / (1.0f + __expf(-gate)));
+                        }
+                        *reinterpret_cast<half4 *>(C + (size_t)m * (N / 2) + n) = o;
+                    }
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+        if (nt0 + t >= ntiles)
+            continue;
+        const int n = (nt0 + t) * 16 + 4 * g;
+        const half4 sc = *reinterpret_cast<const half4 *>(scale + n);
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt) {
+            const int m = mrow0 + 16 * mt;
+            if (m < M) {
+                half4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    o[r] = (_Float16)(acc[t][mt][r] * (float)sc[r]);
+                if (epi == kEpiResidual)
+                    o = o + *reinterpret_cast<const half4 *>(residual + (size_t)m * N + n);  // fp16 add of the rounded product
+                *reinterpret_cast<half4 *>(C + (size_t)m * N + n) = o;
+            }
+        }
+    }
+}
+
+
+// ---------------------------------------------------------------------------
+// Variant with the activations copied global -> LDS by the memory pipeline
+// itself (global_load_lds_dwordx4: no staging registers, no ds_write) into a
+// ring of four k-tile stages, three tiles ahead of the one being multiplied,
+// and the packed weights prefetched two tiles ahead into registers.  One
+// wavefront row (WMW = 1): the block is TM*16 rows x WNW*TN*16 channels, and two
+// such workgroups share a CU with independent barriers.
+//
+// A stage holds TM m-tiles of 2 KiB: [row half b][row r (8)][position (8)] x
+// 16 B, where position p of row (b, r) holds piece p ^ ((r >> 1) | (b << 2)) of
+// the row's eight 16-byte pieces.  One DMA instruction fills 1 KiB (8 rows x
+// 128 B, whole cache lines; the XOR only permutes lanes within a line), and the
+// MFMA operand read of lane (g, j) -- piece 2g+h of row j -- hits 16 distinct
+// 16-byte bank groups per 16 lanes.
+// ---------------------------------------------------------------------------
+constexpr int kDmaStages = 4, kDmaAhead = 3;
+
+__device__ __forceinline__ constexpr int vmcnt_imm(int n)
+{
+    return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14);  // expcnt, lgkmcnt: no wait
+}
+
+template <int WNW, int TM, int TN>
+struct DmaShape {
+    static constexpr int kThreads = 64 * WNW;
+    static constexpr int kBM = TM * 16, kBN = WNW * TN * 16;
+    static constexpr int kStageVec = TM * 128;          // u32x4 per stage
+    static constexpr int kRowGroups = TM * 2;           // DMA instructions per k-tile (8 rows each)
+    static constexpr int kPerWave = kRowGroups / WNW;   // ... per wavefront
+    static_assert(kRowGroups % WNW == 0, "row groups must divide over the wavefronts");
+    static_assert(kDmaStages * kStageVec * 16 <= 65536, "the stage ring must fit 64 KiB");
+};
+
+template <int WNW, int TM, int TN>
+__global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) void w8a16_large_m_dma_kernel(
+    const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
+    _Float16 *__restrict__ C, int M, int N, int K, int m_blocks, int n_blocks,
+    const _Float16 *__restrict__ residual, int epi)
+{
+#if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
+    using S = DmaShape<WNW, TM, TN>;
+    // one array per stage: the compiler tells them apart when it places waits
+    // between the DMA writes and the LDS reads
+    __shared__ u32x4 st0[S::kStageVec], st1[S::kStageVec], st2[S::kStageVec], st3[S::kStageVec];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: feeds scalar offsets and M0
+    const int g = lane >> 4, j = lane & 15;
+    const int ktiles = K >> 6, ntiles = N >> 4;
+
+    const int total = m_blocks * n_blocks;
+    const int per_xcd = (total + 7) / 8;
+    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (tile >= total)
+        return;
+    const int n_blk = tile / m_blocks, m_blk = tile % m_blocks;
+    const int m0 = m_blk * S::kBM;
+    const int nt0 = n_blk * (WNW * TN) + wave * TN;
+
+    // Both operands are addressed through buffer resources: a 32-bit lane offset
+    // plus a scalar offset per tile, and reads past the end (rows >= M, n-tiles
+    // >= N/16) return zeros instead of needing clamped addresses.
+    const size_t a_bytes = (size_t)(M - m0) * K * 2;
+    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<_Float16 *>(A + (size_t)m0 * K), 0, a_bytes > 0xffffffffull ? 0xffffffffu : (unsigned)a_bytes,
+        0x00020000);
+    const __amdgpu_buffer_rsrc_t wrsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4 *>(Wp), 0, (unsigned)((size_t)K * N), 0x00020000);
+    const int woff = lane * 16;
+    unsigned wtile[TN];  // byte offset of the n-tile's first k-tile
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+        wtile[t] = (unsigned)(nt0 + t) * (unsigned)ktiles * 1024u;
+
+    // DMA source of this lane for row group rg = wave * kPerWave + i: row
+    // 8*rg + lane/8, piece (lane%8) ^ swizzle.
+    int aoff[S::kPerWave];
+#pragma unroll
+    for (int i = 0; i < S::kPerWave; ++i) {
+        const int rg = wave * S::kPerWave + i, r = lane >> 3, b = rg & 1;
+        const int piece = (lane & 7) ^ ((r >> 1) | (b << 2));
+        aoff[i] = (8 * rg + r) * K * 2 + piece * 16;
+    }
+    const int swz = ((j & 7) >> 1) | ((j >> 3) << 2);
+    const int rs0 = (j >> 3) * 64 + (j & 7) * 8 + ((2 * g) ^ swz), rs1 = rs0 ^ 1;
+
+    floatx4 acc[TN][TM];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt)
+            acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    u32x4 wraw[2][TN];
+
+    auto dma_tile = [&](u32x4 *stage, int kt) {
+#pragma unroll
+        for (int i = 0; i < S::kPerWave; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(arsrc, stage + (wave * S::kPerWave + i) * 64, 16, aoff[i], kt * 128,
+                                                     0, 0);
+    };
+    auto load_w = [&](u32x4 (&dst)[TN], int kt) {
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+            dst[t] = __builtin_bit_cast(
+                u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, woff, wtile[t] + (unsigned)kt * 1024u, 0));
+    };
+
+    // One k-tile: A from `cur`, raw weights from wb; the DMA for tile kt + 3 goes
+    // to `ahead`, the weights of tile kt + 2 replace wb once it is widened.
+    auto step = [&](const u32x4 *cur, u32x4 *ahead, u32x4 (&wb)[TN], int kt) {
+        dma_tile(ahead, min(kt + kDmaAhead, ktiles - 1));
+        __builtin_amdgcn_sched_barrier(0);
+        half8 w0[TN], w1[TN];
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+            w0[t] = widen8(wb[t].x, wb[t].y);
+            w1[t] = widen8(wb[t].z, wb[t].w);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(wb, min(kt + 2, ktiles - 1));
+        half8 aop[2][2];
+        aop[0][0] = __builtin_bit_cast(half8, cur[rs0]);
+        aop[0][1] = __builtin_bit_cast(half8, cur[rs1]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt) {
+            if (mt + 1 < TM) {
+                aop[(mt + 1) & 1][0] = __builtin_bit_cast(half8, cur[(mt + 1) * 128 + rs0]);
+                aop[(mt + 1) & 1][1] = __builtin_bit_cast(half8, cur[(mt + 1) * 128 + rs1]);
+            }
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0[t], aop[mt & 1][0], acc[t][mt], 0, 0, 0);
+                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1[t], aop[mt & 1][1], acc[t][mt], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt) {
+            if (mt + 1 < TM)
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // 2 LDS reads
+            __builtin_amdgcn_sched_group_barrier(0x008, 2 * TN, 0);  // 2*TN MFMA
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // The DMA of tile kt+1 (issued two steps ago) must have landed before any
+        // wavefront reads it: everything older than the loads of the last two steps
+        // (2 x (kPerWave DMA + TN weight loads)), then the barrier.
+        // (A plain __syncthreads() would drain every outstanding load here: its
+        // release fence waits for all DMA writes, including the ones just issued.)
+        static_assert(2 * (S::kPerWave + TN) == 16, "the wait count below is written out as a literal");
+        asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
+    };
+
+    // prologue: tiles 0..2 into stages 0..2, weights of tiles 0 and 1
+    load_w(wraw[0], 0);
+    dma_tile(st0, 0);
+    load_w(wraw[1], min(1, ktiles - 1));
+    dma_tile(st1, min(1, ktiles - 1));
+    dma_tile(st2, min(2, ktiles - 1));
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    __syncthreads();
+
+    int kt = 0;
+    for (; kt + 4 <= ktiles; kt += 4) {
+        step(st0, st3, wraw[0], kt);
+        step(st1, st0, wraw[1], kt + 1);
+        step(st2, st1, wraw[0], kt + 2);
+        step(st3, st2, wraw[1], kt + 3);
+    }
+    if (kt < ktiles)
+        step(st0, st3, wraw[0], kt);
+    if (kt + 1 < ktiles)
+        step(st1, st0, wraw[1], kt + 1);
+    if (kt + 2 < ktiles)
+        step(st2, st1, wraw[0], kt + 2);
+
+    // acc[t][mt][r] of lane (g, j): row m0 + 16*mt + j, channel 16*(nt0+t) + 4*g + r
+    const int mrow0 = m0 + j;
+    if (epi == kEpiSwiglu) {
+        if constexpr (TN % 2 == 0) {
+#pragma unroll
+            for (int t = 0; t < TN; t += 2) {
+                if (nt0 + t + 1 >= ntiles)
+                    continue;
+                const half4 sg = *reinterpret_cast<const half4 *>(scale + (nt0 + t) * 16 + 4 * g);
+                const half4 su = *reinterpret_cast<const half4 *>(scale + (nt0 + t + 1) * 16 + 4 * g);
+                const int n = ((nt0 + t) / 2) * 16 + 4 * g;
+#pragma unroll
+                for (int mt = 0; mt < TM; ++mt) {
+                    const int m = mrow0 + 16 * mt;
+                    if (m < M) {
+                        half4 o;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const float gate = (float)(_Float16)(acc[t][mt][r] * (float)sg[r]);
+                            const float up = (float)(_Float16)(acc[t + 1][mt][r] * (float)su[r]);
+                            o[r] = (_Float16)(up * gate / (1.0f + __expf(-gate)));
+                        }
+                        *reinterpret_cast<half4 *>(C + (size_t)m * (N / 2) + n) = o;
+                    }
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+        if (nt0 + t >= ntiles)
+            continue;
+        const int n = (nt0 + t) * 16 + 4 * g;
+        const half4 sc = *reinterpret_cast<const half4 *>(scale + n);
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt) {
+            const int m = mrow0 + 16 * mt;
+            if (m < M) {
+                half4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    o[r] = (_Float16)(acc[t][mt][r] * (float)sc[r]);
+                if (epi == kEpiResidual)
+                    o = o + *reinterpret_cast<const half4 *>(residual + (size_t)m * N + n);
+                *reinterpret_cast<half4 *>(C + (size_t)m * N + n) = o;
+            }
+        }
+    }
+#endif
+}
+
+template <int WNW, int TM, int TN>
+int launch_large_m_dma(const GemmArgs &a)
+{
+    using S = DmaShape<WNW, TM, TN>;
+    const int m_blocks = (a.M + S::kBM - 1) / S::kBM, n_blocks = (a.N + S::kBN - 1) / S::kBN;
+    const int grid = ((m_blocks * n_blocks + 7) / 8) * 8;
+    hipLaunchKernelGGL((w8a16_large_m_dma_kernel<WNW, TM, TN>), dim3(grid), dim3(S::kThreads), 0, a.st, a.A, a.Wp,
+                       a.scale, a.C, a.M, a.N, a.K, m_blocks, n_blocks, a.residual, a.epi);
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
+template <int WMW, int WNW, int TM, int TN>
+int launch_large_m(const GemmArgs &a)
+{
+    using S = LmShape<WMW, WNW, TM, TN>;
+    const int m_blocks = (a.M + S::kBM - 1) / S::kBM, n_blocks = (a.N + S::kBN - 1) / S::kBN;
+    const int grid = ((m_blocks * n_blocks + 7) / 8) * 8;
+    hipLaunchKernelGGL((w8a16_large_m_kernel<WMW, WNW, TM, TN>), dim3(grid), dim3(S::kThreads), 0, a.st, a.A, a.Wp,
+                       a.scale, a.C, a.M, a.N, a.K, m_blocks, n_blocks, a.residual, a.epi);
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
+struct LargeMConfig {
+    int wmw, wnw, tm, tn;  // wmw = 0: the DMA kernel (one wavefront row)
+};
+
+// Shape -> tile.  Measured on MI355X (M = 129 .. 8192, LLaMA-7B and Baichuan-13B shapes):
+//   128 x 256 (DMA kernel, two workgroups per CU) is the fastest tile once it yields
+//     a few hundred workgroups;
+//   128 x 320 (8 wavefronts) wins when it divides the problem into whole rounds of
+//     256 workgroups where 128 x 256 leaves a CU with two tiles against one elsewhere
+//     (M = 2048, N = 5120: 256 tiles instead of 320);
+//   64 x 128 and 32 x 128 keep the chip occupied for M in the hundreds, where the
+//     k-loop latency of the few large tiles would dominate.
+LargeMConfig pick_large_m(int M, int N, int epi)
+{
+    auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    const int big = wgs(128, 256);
+    if (big >= 320) {
+        if (epi != kEpiSwiglu) {  // 128 x 320 holds 5 n-tiles per wavefront: no (gate, up) pairs
+            const double cost_big = 2.0 * ((big + 511) / 512);
+            const double cost_320 = ((wgs(128, 320) + 255) / 256) * (320.0 / 256.0) / 0.9;
+            if (cost_320 < cost_big)
+                return LargeMConfig{2, 4, 4, 5};
+        }
+        return LargeMConfig{0, 4, 8, 4};
+    }
+    if (wgs(64, 128) >= 300)
+        return LargeMConfig{1, 4, 4, 2};
+    return LargeMConfig{1, 4, 2, 2};
+}
+
+}  // namespace
+
+int eet::run_large_m(const GemmArgs &a)
+{
+    // the kernels address A rows and the packed weights with 32-bit byte offsets
+    if ((size_t)a.K * a.N >= (1ull << 31) || (size_t)a.K * 2 * 256 >= (1ull << 31))
+        return eet::fail(EET_ERR_UNSUPPORTED_SHAPE, "eet_gemm_w8a16: K x N = %d x %d exceeds the 2 GiB weight limit",
+                         a.K, a.N);
+    LargeMConfig c = pick_large_m(a.M, a.N, a.epi);
+    if (const char *env = std::getenv("EET_GEMM_LARGE_M_TILE")) {  // "wmw,wnw,tm,tn": tuning override
+        LargeMConfig e = c;
+        if (sscanf(env, "%d,%d,%d,%d", &e.wmw, &e.wnw, &e.tm, &e.tn) == 4 && (a.epi != kEpiSwiglu || e.tn % 2 == 0))
+            c = e;
+    }
+    if (c.wmw == 0 && c.wnw == 4 && c.tm == 8 && c.tn == 4)
+        return launch_large_m_dma<4, 8, 4>(a);
+#define EET_LM_CASE(A_, B_, C_, D_)                                      \
+    if (c.wmw == A_ && c.wnw == B_ && c.tm == C_ && c.tn == D_)         \
+        return launch_large_m<A_, B_, C_, D_>(a);
+    EET_LM_CASE(1, 4, 8, 4)
+    EET_LM_CASE(2, 4, 4, 5)
+    EET_LM_CASE(1, 4, 4, 2)
+    EET_LM_CASE(1, 4, 2, 2)
+#undef EET_LM_CASE
+    return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no large-M kernel for tile %d,%d,%d,%d", c.wmw, c.wnw,
+                     c.tm, c.tn);
+}

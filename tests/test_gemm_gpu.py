@@ -96,6 +96,31 @@ def test_large_m_path(gpu):
         assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32), what=f"M={M}")
 
 
+LARGE_M_TILES = ["0,4,8,4", "1,4,8,4", "2,4,4,5", "1,4,4,2", "1,4,2,2"]
+
+
+@pytest.mark.parametrize("tile", LARGE_M_TILES)
+def test_large_m_tiles(gpu, monkeypatch, tile):
+    """Every large-M kernel variant (selected with the tuning override), on ragged M / N edges and on
+    k-loops of 1..9 tiles (prologue, unrolled body and tail of the software pipeline)."""
+    monkeypatch.setenv("EET_GEMM_LARGE_M_TILE", tile)
+    for (M, K, N) in [(129, 64, 48), (300, 128, 272), (257, 192, 720), (200, 256, 336), (512, 320, 256),
+                      (130, 448, 64), (333, 576, 1040)]:
+        x, u, p, s = make(M, K, N, M + K + N)
+        c = gemm(x.to(gpu), p.to(gpu), s.to(gpu), M, N, K)
+        assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32),
+                     what=f"tile {tile} M={M} K={K} N={N}")
+
+
+@pytest.mark.parametrize("M,K,N,tile", [(1024, 256, 12288, "0,4,8,4"), (2048, 256, 5120, "2,4,4,5"),
+                                        (512, 256, 4096, "1,4,4,2"), (256, 256, 1024, "1,4,2,2")])
+def test_large_m_dispatch(gpu, M, K, N, tile):
+    """Shapes on which the dispatcher itself picks each tile (named for the record) -- no override."""
+    x, u, p, s = make(M, K, N, 77)
+    c = gemm(x.to(gpu), p.to(gpu), s.to(gpu), M, N, K)
+    assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32), what=tile)
+
+
 def test_full_size_linearity(gpu):
     """Size-independent property at a BASELINE shape: gemm(a + b) == gemm(a) + gemm(b) within fp16 rounding,
     and doubling the scales doubles the output exactly."""
@@ -153,6 +178,33 @@ def test_swiglu_epilogue(gpu, M, K, F):
     uu, pu, su = eet_amd.quant_weights(wu, torch.int8, True)
     w01, s01 = interleave_gate_up(pg, sg, pu, su)
     got = fused(x.to(gpu), w01.to(gpu), s01.to(gpu), M, 2 * F, K, 2).cpu().numpy()
+    want = O.swiglu(O.dequant_matmul(x.numpy(), ug.numpy(), sg.numpy()),
+                    O.dequant_matmul(x.numpy(), uu.numpy(), su.numpy()))
+    assert_close(got, want, rtol=1e-2, atol=1e-3)
+
+
+@pytest.mark.parametrize("tile", LARGE_M_TILES)
+def test_large_m_tile_epilogues(gpu, monkeypatch, tile):
+    """Residual and SwiGLU epilogues of every large-M kernel variant (5 n-tiles per wavefront cannot
+    pair gate / up tiles: there the override is ignored for SwiGLU and the dispatcher's own choice runs)."""
+    from eet_amd.ops import interleave_gate_up
+    monkeypatch.setenv("EET_GEMM_LARGE_M_TILE", tile)
+    M, K, N = 270, 320, 592
+    x, u, p, s = make(M, K, N, 5)
+    res = torch.randn(M, N, generator=torch.Generator().manual_seed(M)).half()
+    xd, pd, sd, rd = x.to(gpu), p.to(gpu), s.to(gpu), res.to(gpu)
+    got = fused(xd, pd, sd, M, N, K, 1, rd).cpu()
+    assert torch.equal(got, gemm(xd, pd, sd, M, N, K).cpu() + res)
+    assert_close(got.numpy(), O.residual_add(O.dequant_matmul(x.numpy(), u.numpy(), s.numpy()), res.numpy()),
+                 rtol=1e-2, atol=2e-3)
+    F = 336
+    g = torch.Generator().manual_seed(F)
+    wg = (torch.randn(K, F, generator=g) * 0.02).half()
+    wu = (torch.randn(K, F, generator=g) * 0.02).half()
+    ug, pg, sg = eet_amd.quant_weights(wg, torch.int8, True)
+    uu, pu, su = eet_amd.quant_weights(wu, torch.int8, True)
+    w01, s01 = interleave_gate_up(pg, sg, pu, su)
+    got = fused(xd, w01.to(gpu), s01.to(gpu), M, 2 * F, K, 2).cpu().numpy()
     want = O.swiglu(O.dequant_matmul(x.numpy(), ug.numpy(), sg.numpy()),
                     O.dequant_matmul(x.numpy(), uu.numpy(), su.numpy()))
     assert_close(got, want, rtol=1e-2, atol=1e-3)

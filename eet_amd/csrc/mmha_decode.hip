@@ -10,14 +10,13 @@
 //
 // HBM-bound: K and V rows (dh halves, contiguous) are each read exactly once
 // with 128-bit loads.  The cache is [B_cap][H][T_cap][dh], so one (b, h) pair
-// streams one contiguous range.  The time axis is split over `nsplit`
-// workgroups per (b, h) so that a few hundred heads still fill 256 CUs
-// (the reference runs one block per head); every workgroup produces an
+// streams one contiguous range.  A workgroup of 512 lanes serves one (b, h):
+// every group of dh/8 lanes streams its own rows with a running softmax and a
+// small ring of rows in flight, and the streams meet once in LDS.  Only when
+// there are fewer (b, h) pairs than CUs is the time axis split over `nsplit`
+// workgroups (the reference runs one block per head); each then writes an
 // un-normalised partial (max, sum, acc[dh]) and a second small kernel merges
-// them.  With nsplit == 1 the first kernel writes the context itself.
-// Inside a workgroup every group of dh/8 lanes streams its own rows with a
-// running softmax, K and V rows requested together several rows deep; there
-// is no per-launch limit on step.
+// them.  There is no per-launch limit on step.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -31,8 +30,6 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kThreads = 256;
-
 __device__ __forceinline__ float dot8(const u32x4 &a, const u32x4 &b)
 {
     const half8 ha = __builtin_bit_cast(half8, a), hb = __builtin_bit_cast(half8, b);
@@ -44,12 +41,6 @@ __device__ __forceinline__ float dot8(const u32x4 &a, const u32x4 &b)
     return s;
 }
 
-// Decode streams every cache row exactly once: non-temporal loads.
-__device__ __forceinline__ u32x4 load_row16(const u32x4 *p)
-{
-    return __builtin_nontemporal_load(p);
-}
-
 template <int WIDTH>
 __device__ __forceinline__ float group_sum(float v)
 {
@@ -57,25 +48,6 @@ __device__ __forceinline__ float group_sum(float v)
     for (int off = WIDTH / 2; off > 0; off >>= 1)
         v += __shfl_xor(v, off, 64);
     return v;
-}
-
-__device__ __forceinline__ float block_reduce(float v, bool is_max, float *scratch)
-{
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        float o = __shfl_xor(v, off, 64);
-        v = is_max ? fmaxf(v, o) : v + o;
-    }
-    if (lane == 0)
-        scratch[wave] = v;
-    __syncthreads();
-    float r = scratch[0];
-#pragma unroll
-    for (int w = 1; w < kThreads / 64; ++w)
-        r = is_max ? fmaxf(r, scratch[w]) : r + scratch[w];
-    __syncthreads();
-    return r;
 }
 
 // NeoX rotary on one 8-element slice.  x holds elements d = 8*sub .. 8*sub+7 of
@@ -100,15 +72,15 @@ __device__ __forceinline__ u32x4 rotate8(const u32x4 &x, const u32x4 &y, int sub
 
 // DH: head size.  LPR = DH/8 lanes cover one row with one 16-byte load each.
 // One query per (b, h) attends rows [0, step); grid = (B*H, nsplit).
-template <int DH, int UN>
-__global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
+template <int DH, int UN, int THREADS>
+__global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_new, const _Float16 *__restrict__ v_new,
     long qkv_stride, _Float16 *__restrict__ k_cache, _Float16 *__restrict__ v_cache, _Float16 *__restrict__ ctx,
     const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, float *__restrict__ partial, int H,
     int step, int T_cap, int nsplit, float scale, const float *__restrict__ rope_row)
 {
     constexpr int LPR = DH / 8;            // lanes per row
-    constexpr int RPB = kThreads / LPR;    // row streams of the block (one per group of LPR lanes)
+    constexpr int RPB = THREADS / LPR;    // row streams of the block (one per group of LPR lanes)
     __shared__ float accs[RPB][DH + 1];
     __shared__ float stream_m[RPB], stream_l[RPB];
 
@@ -164,42 +136,62 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
     }
 
     // Every group of LPR lanes walks its own stream of rows (rs, rs + RPB, ...)
-    // with a running softmax (max m, sum l, un-normalised acc): K and V rows are
-    // requested together, UN rows deep, and nothing synchronises the workgroup
-    // until the streams are merged at the end.
+    // with a running softmax (max m, sum l, un-normalised acc).  The K and V rows
+    // (and the ALiBi term) of a stream sit in a ring of UN register slots: row i
+    // is consumed from slot i % UN and the request for row i + UN goes out in its
+    // place, so UN rows per stream stay in flight from the first row to the last
+    // and nothing synchronises the workgroup until the streams are merged.
+    // The cache range of this workgroup is addressed through buffer resources
+    // whose size is exactly its n rows: requests past the end return zeros
+    // without touching memory, which keeps the loop free of branches around loads.
+#if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
+    const unsigned range_bytes = (unsigned)n * (unsigned)(DH * 2);
+    const __amdgpu_buffer_rsrc_t krs =
+        __builtin_amdgcn_make_buffer_rsrc(kc + (size_t)t0 * DH, 0, range_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrs =
+        __builtin_amdgcn_make_buffer_rsrc(vc + (size_t)t0 * DH, 0, range_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ars = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<_Float16 *>(alibi ? alibi + (size_t)h * alibi_ld + t0 : q), 0, alibi ? (unsigned)n * 2u : 0u,
+        0x00020000);
+    constexpr int kStream = 2;  // aux bits of a buffer load: non-temporal (every row is read exactly once)
+    auto row_off = [&](int i) { return (unsigned)((rs + i * RPB) * (DH * 2) + sub * 16); };
+    // The first pass of the loop (i0 = -UN) only fills the ring: there is no separate
+    // prologue, so the wait before each slot is the same on every pass (all but the
+    // UN-1 newer slots' requests) instead of the merge with a differently ordered
+    // prologue, which drained the ring once per pass.
+    u32x4 kv[UN], vv[UN];
+    unsigned short ab[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+        kv[u] = u32x4{0, 0, 0, 0};
+        vv[u] = u32x4{0, 0, 0, 0};
+        ab[u] = 0;
+    }
     float m_run = -INFINITY, l_run = 0.f;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int r0 = rs; r0 < n; r0 += RPB * UN) {
-        u32x4 kv[UN], vv[UN];
+    const int iters = (n + RPB - 1) / RPB;  // the same for every stream of the workgroup
+    for (int i0 = -UN; i0 < iters; i0 += UN) {
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const int r = r0 + u * RPB;
-            if (r < n)
-                kv[u] = (r == r_last)
-                            ? knew
-                            : load_row16(reinterpret_cast<const u32x4 *>(kc + (size_t)(t0 + r) * DH) + sub);
-        }
-#pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const int r = r0 + u * RPB;
-            if (r < n)
-                vv[u] = (r == r_last)
-                            ? vnew
-                            : load_row16(reinterpret_cast<const u32x4 *>(vc + (size_t)(t0 + r) * DH) + sub);
-        }
-#pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const int r = r0 + u * RPB;  // the same for all LPR lanes of a group
-            float d = (r < n) ? dot8(qv, kv[u]) : 0.f;
-            d = group_sum<LPR>(d) * scale;
-            if (r < n) {
-                if (alibi)
-                    d += (float)alibi[(size_t)h * alibi_ld + t0 + r];
+            const int r = rs + (i0 + u) * RPB;  // the same for all LPR lanes of a group
+            u32x4 kcur = kv[u], vcur = vv[u];
+            const unsigned short acur = ab[u];
+            kv[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(krs, row_off(i0 + u + UN), 0, kStream));
+            vv[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(vrs, row_off(i0 + u + UN), 0, kStream));
+            ab[u] = __builtin_amdgcn_raw_buffer_load_b16(ars, (unsigned)((rs + (i0 + u + UN) * RPB) * 2), 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (r == r_last) {  // the row being appended by this launch is still in registers
+                kcur = knew;
+                vcur = vnew;
+            }
+            float d = group_sum<LPR>(dot8(qv, kcur)) * scale;
+            if (r >= 0 && r < n) {
+                d += (float)__builtin_bit_cast(_Float16, acur);  // 0 without ALiBi
                 const float m_new = fmaxf(m_run, d);
                 const float c = __expf(m_run - m_new);  // 0 on the first row (m_run = -inf)
                 const float p = __expf(d - m_new);
                 l_run = l_run * c + p;
-                const half8 hv = __builtin_bit_cast(half8, vv[u]);
+                const half8 hv = __builtin_bit_cast(half8, vcur);
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
                     acc[e] = acc[e] * c + p * (float)hv[e];
@@ -207,6 +199,10 @@ __global__ __launch_bounds__(kThreads) void mmha_decode_split_kernel(
             }
         }
     }
+#else
+    float m_run = -INFINITY, l_run = 0.f;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#endif
 
     // Merge the RPB streams of the workgroup.
 #pragma unroll
@@ -263,35 +259,58 @@ __global__ __launch_bounds__(DH) void mmha_decode_merge_kernel(const float *__re
     ctx[(size_t)bh * DH + tid] = (_Float16)(acc / (sum + 1e-6f));
 }
 
-int pick_nsplit(int BH, int step)
+// How a launch is cut: `nsplit` workgroups of `threads` lanes per (b, h), each
+// stream with a ring of `ring` rows.  Measured on MI355X (B*H = 256 at step ~1100
+// and B*H = 1280 at step ~2200, 256 / 512 / 1024 lanes x 1..16 splits x rings of
+// 2, 4, 8): 512 lanes (32 row streams at dh = 128) and no split is the fastest on
+// both -- 25 us and 211 us, against 27-36 us and 217-224 us for the other widths --
+// and shallow rings beat deep ones (more resident wavefronts matter more than
+// more rows in flight per stream).  With fewer than 256 (b, h) pairs the time
+// axis is split until there is one workgroup per CU, as long as a split keeps
+// 256 rows; a short cache (under 8 rows per stream) takes 256-lane workgroups.
+struct Plan {
+    int threads, nsplit, ring;
+};
+
+Plan pick_plan(int BH, int dh, int step)
 {
-    static const int forced = [] {
-        const char *e = std::getenv("EET_MMHA_NSPLIT");  // tuning override
+    // tuning overrides, read on every call (a getenv is noise next to a launch)
+    auto env_int = [](const char *name) {
+        const char *e = std::getenv(name);
         return e ? atoi(e) : 0;
-    }();
-    if (forced > 0)
-        return forced;
-    // Measured on MI355X (B*H = 256 at step ~1100 and B*H = 1280 at step ~2200):
-    // up to ~4096 workgroups, but no fewer than 256 rows each.
-    int want = (4096 + BH - 1) / BH;
-    int by_rows = step / 256;
-    int ns = want < by_rows ? want : by_rows;
-    return ns < 1 ? 1 : ns;
+    };
+    const int forced_ns = env_int("EET_MMHA_NSPLIT"), forced_threads = env_int("EET_MMHA_THREADS");
+    const int forced_ring = env_int("EET_MMHA_UNROLL");
+    Plan p{512, 1, 4};
+    const int want = (256 + BH - 1) / BH, by_rows = step / 256;
+    p.nsplit = want < by_rows ? want : by_rows;
+    if (p.nsplit < 1)
+        p.nsplit = 1;
+    if (forced_ns > 0)
+        p.nsplit = forced_ns;
+    if (forced_threads == 256 || forced_threads == 512 || forced_threads == 1024)
+        p.threads = forced_threads;
+    else if (step / p.nsplit / (p.threads / (dh / 8)) < 8)
+        p.threads = 256;
+    const int rows_per_stream = step / p.nsplit / (p.threads / (dh / 8));
+    p.ring = rows_per_stream < 64 ? 2 : 4;
+    if (forced_ring == 2 || forced_ring == 4 || forced_ring == 8)
+        p.ring = forced_ring;
+    return p;
 }
 
-template <int DH>
-int launch(const void *q, const void *k, const void *v, long qkv_stride, void *kc, void *vc, void *ctx,
-           const void *alibi, const int64_t *pad, int B, int H, int step, int T_cap, void *ws, int nsplit,
-           const float *rope_row, hipStream_t st)
+template <int DH, int THREADS>
+int launch_split(const void *q, const void *k, const void *v, long qkv_stride, void *kc, void *vc, void *ctx,
+                 const void *alibi, const int64_t *pad, int B, int H, int step, int T_cap, void *ws, Plan plan,
+                 const float *rope_row, hipStream_t st)
 {
     const float scale = (float)(_Float16)(1.0f / sqrtf((float)DH));
+    const int nsplit = plan.nsplit;
     dim3 grid(B * H, nsplit);
-    static const int unroll = [] {
-        const char *e = std::getenv("EET_MMHA_UNROLL");
-        return e ? atoi(e) : 8;
-    }();
-    auto kern = (unroll == 4) ? mmha_decode_split_kernel<DH, 4> : mmha_decode_split_kernel<DH, 8>;
-    hipLaunchKernelGGL(kern, grid, dim3(kThreads), 0, st,
+    auto kern = (plan.ring == 8)   ? mmha_decode_split_kernel<DH, 8, THREADS>
+                : (plan.ring == 2) ? mmha_decode_split_kernel<DH, 2, THREADS>
+                                   : mmha_decode_split_kernel<DH, 4, THREADS>;
+    hipLaunchKernelGGL(kern, grid, dim3(THREADS), 0, st,
                        static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(k),
                        static_cast<const _Float16 *>(v), qkv_stride, static_cast<_Float16 *>(kc),
                        static_cast<_Float16 *>(vc), static_cast<_Float16 *>(ctx),
@@ -304,6 +323,21 @@ int launch(const void *q, const void *k, const void *v, long qkv_stride, void *k
         EET_HIP_CHECK(hipGetLastError());
     }
     return EET_OK;
+}
+
+template <int DH>
+int launch(const void *q, const void *k, const void *v, long qkv_stride, void *kc, void *vc, void *ctx,
+           const void *alibi, const int64_t *pad, int B, int H, int step, int T_cap, void *ws, Plan plan,
+           const float *rope_row, hipStream_t st)
+{
+    if (plan.threads == 1024)
+        return launch_split<DH, 1024>(q, k, v, qkv_stride, kc, vc, ctx, alibi, pad, B, H, step, T_cap, ws, plan,
+                                      rope_row, st);
+    if (plan.threads == 512)
+        return launch_split<DH, 512>(q, k, v, qkv_stride, kc, vc, ctx, alibi, pad, B, H, step, T_cap, ws, plan,
+                                     rope_row, st);
+    return launch_split<DH, 256>(q, k, v, qkv_stride, kc, vc, ctx, alibi, pad, B, H, step, T_cap, ws, plan, rope_row,
+                                 st);
 }
 
 }  // namespace
@@ -338,7 +372,7 @@ extern "C" size_t eet_mmha_decode_workspace(int B, int H, int dh, int step)
 {
     if (B <= 0 || H <= 0 || dh <= 0 || step <= 0)
         return 0;
-    const int ns = pick_nsplit(B * H, step);
+    const int ns = pick_plan(B * H, dh, step).nsplit;
     return ns > 1 ? (size_t)B * H * ns * (dh + 2) * sizeof(float) : 0;
 }
 
@@ -360,7 +394,7 @@ extern "C" int eet_mmha_decode(const void *q, const void *k, const void *v, long
                 "eet_mmha_decode: qkv_stride must be a non-negative multiple of 8");
     EET_REQUIRE(rope_cos_sin == nullptr || k != nullptr, EET_ERR_INVALID_ARGUMENT,
                 "eet_mmha_decode: a rotary row needs the new k, v (it rotates q and the appended k)");
-    const int ns = pick_nsplit(B * H, step);
+    const Plan ns = pick_plan(B * H, dh, step);
     const size_t need = eet_mmha_decode_workspace(B, H, dh, step);
     EET_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), EET_ERR_WORKSPACE,
                 "eet_mmha_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);

@@ -49,6 +49,29 @@ def test_against_oracle(gpu, B, H, dh, step, cap, use_pad, use_alibi):
     assert np.array_equal(kcd.cpu().numpy(), kcn) and np.array_equal(vcd.cpu().numpy(), vcn)
 
 
+@pytest.mark.parametrize("threads", [256, 512, 1024])
+@pytest.mark.parametrize("ring", [2, 4, 8])
+@pytest.mark.parametrize("nsplit", [1, 3])
+def test_every_launch_shape(gpu, monkeypatch, threads, ring, nsplit):
+    """Every workgroup width / ring depth / split count the kernel is instantiated for (selected with the
+    tuning overrides), with padding, ALiBi, the fused rotary append and a ragged last pass of the ring."""
+    monkeypatch.setenv("EET_MMHA_THREADS", str(threads))
+    monkeypatch.setenv("EET_MMHA_UNROLL", str(ring))
+    monkeypatch.setenv("EET_MMHA_NSPLIT", str(nsplit))
+    for (B, H, dh, step, use_pad, use_alibi) in [(2, 3, 128, 333, True, False), (2, 2, 64, 1207, False, True),
+                                                 (1, 2, 32, 45, True, True), (3, 2, 128, 3, False, False)]:
+        cap = step + 3
+        q, k, v, kc, vc, pad, alibi = case(B, H, dh, step, cap, step + threads, use_pad, use_alibi)
+        kcn, vcn = kc.numpy().copy(), vc.numpy().copy()
+        want = O.decode_attention(q.numpy(), k.numpy(), v.numpy(), kcn, vcn, step,
+                                  pad.numpy() if use_pad else None, alibi.numpy() if use_alibi else None)
+        kcd, vcd = kc.to(gpu), vc.to(gpu)
+        ctx = mmha(q.to(gpu), k.to(gpu), v.to(gpu), kcd, vcd, step, pad.to(gpu) if use_pad else None,
+                   alibi.to(gpu) if use_alibi else None)
+        assert_close(ctx.cpu().numpy(), want, what=f"ctx B={B} H={H} dh={dh} step={step}")
+        assert np.array_equal(kcd.cpu().numpy(), kcn) and np.array_equal(vcd.cpu().numpy(), vcn)
+
+
 def test_known_answers(gpu):
     B, H, dh, cap = 2, 3, 128, 300
     q, k, v, kc, vc, _, _ = case(B, H, dh, 1, cap, 5)

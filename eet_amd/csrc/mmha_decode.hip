@@ -109,9 +109,12 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
     // `sub` of the new k and v) and writes it to the cache on the side; no
     // other workgroup of this launch reads that row, so no fence is needed.
     // With a rotary row given, k is rotated on the way in (pairs d, d + DH/2).
+    // (A sequence whose padding covers the new token too has no such row; split 0
+    // appends it all the same, as the reference does, and gives it no weight.)
     const bool own_last = k_new != nullptr && step - 1 >= t0 && step - 1 < t1;
+    const bool append = own_last || (k_new != nullptr && span == 0 && split == 0);
     u32x4 knew = {0, 0, 0, 0}, vnew = {0, 0, 0, 0};
-    if (own_last) {
+    if (append) {
         knew = *reinterpret_cast<const u32x4 *>(k_new + qoff + sub * 8);
         if (rope_row != nullptr) {
             const u32x4 ky = *reinterpret_cast<const u32x4 *>(k_new + qoff + (sub ^ (LPR / 2)) * 8);

@@ -223,3 +223,30 @@ def test_beam_search_reorder(gpu, alibi):
     with pytest.raises(RuntimeError, match="reorder_state"):
         attn.forward(x1.to(gpu), e, torch.tensor([0, 1, 2], dtype=torch.int32, device=gpu), True, True, False,
                      D.alibi_mask(cfg.heads, step + 1)[:, -1:, :].contiguous().to(gpu) if alibi else torch.empty(0))
+
+
+@pytest.mark.parametrize("alibi", [False, True])
+def test_left_padded_batch(gpu, alibi):
+    """attention_mask with left padding -> pre_padding_len (modeling_llama.py:276-279): prefill and
+    three decode steps against the oracle decoder; the last position of every sequence is a real token."""
+    cfg = tiny_cfg(alibi)
+    sd, raw = D.random_state_dict(cfg, seed=21)
+    sd["lm_head.weight"] = sd["lm_head.weight"] * 8
+    model = D.Int8Decoder(cfg, sd, device="cuda:0")
+    ref = oracle_decoder(cfg, sd, raw)
+    g = torch.Generator().manual_seed(8)
+    B, S = 3, 10
+    ids = torch.randint(0, cfg.vocab, (B, S), generator=g)
+    pads = [0, 4, 7]
+    mask = torch.ones(B, S, dtype=torch.long)
+    for b, p in enumerate(pads):
+        mask[b, :p] = 0
+    pad_np = np.array(pads, dtype=np.int64)
+    logits = ref.step(ids.numpy(), True, pad_np)
+    got = model.logits(ids.to(gpu), True, mask.to(gpu)).float().cpu().numpy()[:, 0]
+    for t in range(3):
+        assert_close(got, logits, 3e-2, 3e-2, f"logits step {t}")
+        nxt = logits.argmax(-1)
+        logits = ref.step(nxt[:, None], False, pad_np)
+        got = model.logits(torch.from_numpy(nxt)[:, None].to(gpu), False, mask.to(gpu)).float().cpu().numpy()[:, 0]
+    assert_close(got, logits, 3e-2, 3e-2, "logits last step")

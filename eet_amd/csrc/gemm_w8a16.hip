@@ -366,6 +366,7 @@ int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a)
         // the launch shapes pick_small_m can return
         EET_CASE_RMS(1, 8, 2) EET_CASE_RMS(1, 16, 2) EET_CASE_RMS(1, 16, 1)
         EET_CASE_RMS(2, 8, 2) EET_CASE_RMS(2, 8, 1) EET_CASE_RMS(3, 8, 1)
+        EET_CASE_RMS(4, 8, 1)
         return eet::fail(EET_ERR_INVALID_ARGUMENT,
                          "eet_gemm_w8a16_fused: no RMSnorm-prologue kernel for nt=%d waves=%d u=%d", cfg.nt,
                          cfg.waves, cfg.u);
@@ -380,12 +381,19 @@ int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a)
                      cfg.nt, cfg.waves, cfg.u, a.M);
 }
 
-// Shape -> launch shape.  Measured on MI355X (LLaMA-7B shapes, M = 1..32).
-// Every workgroup reads all M x K activations once, so with enough n-tiles
-// three of them per workgroup (activation operand reused three times) win as
-// soon as M > 4; with few n-tiles one per workgroup is needed to occupy the
-// 256 CUs, and 16 wavefronts keep enough loads in flight.  The SwiGLU epilogue
-// needs an even number of n-tiles per workgroup (gate / up pairs).
+// Shape -> launch shape: the number of n-tiles per workgroup (NT) that minimises
+//   load * (1 + 0.37 * M / (8 * NT)) * (1 + 0.1 / min(4, workgroups / 256))
+// where load = ceil(workgroups / 256) * NT is the number of n-tiles the busiest CU
+// streams (the kernel is HBM-bound and a CU streams at a fixed rate, so a launch
+// of 320 workgroups costs as much as one of 512), the second factor the
+// activation traffic (every workgroup reads all M x K activations; they come
+// from L2 at about 0.37 of the cost of an HBM byte, 1 KiB per 8 rows and k-tile
+// against NT KiB of weights), the third a mild preference for several
+// workgroups per CU.  Fitted to sweeps over NT = 1..4 on MI355X at M = 8, 16, 32 on
+// the LLaMA-7B shapes (N/16 = 768, 256, 1376, 256 n-tiles) and the Baichuan-13B
+// shapes (960, 320, 1712, 320), whose order it reproduces.  The SwiGLU epilogue
+// needs an even NT (gate / up pairs).  One n-tile per workgroup runs with 16
+// wavefronts when there are few workgroups (more loads in flight per CU).
 SmallMConfig pick_small_m(int M, int N, int K, int epi, bool rms)
 {
     const char *env = std::getenv("EET_GEMM_SMALL_M_CONFIG");  // "nt,waves,u": tuning override
@@ -396,13 +404,27 @@ SmallMConfig pick_small_m(int M, int N, int K, int epi, bool rms)
     }
     const int ntiles = N / 16;
     (void)K;
-    if (epi == kEpiSwiglu)  // with the RMSnorm prologue U = 2 costs a resident workgroup (146 registers): 20.4 us against 17.9 us
-        return (M > 16 || rms) ? SmallMConfig{2, 8, 1} : SmallMConfig{2, 8, 2};
-    if (ntiles >= 600)
-        return (M <= 4) ? SmallMConfig{1, 8, 2} : SmallMConfig{3, 8, 1};
-    if (ntiles >= 400)
-        return (M > 16) ? SmallMConfig{2, 8, 1} : SmallMConfig{2, 8, 2};
-    return (M > 16) ? SmallMConfig{1, 16, 1} : SmallMConfig{1, 16, 2};
+    int best_nt = 0;
+    double best = 0.0;
+    for (int nt = (epi == kEpiSwiglu) ? 2 : 1; nt <= 4; nt += (epi == kEpiSwiglu) ? 2 : 1) {
+        const int wgs = (ntiles + nt - 1) / nt;
+        const double load = (double)((wgs + 255) / 256) * nt;
+        const double per_cu = wgs / 256.0 < 4.0 ? wgs / 256.0 : 4.0;
+        const double cost = load * (1.0 + 0.37 * M / (8.0 * nt)) * (1.0 + 0.1 / per_cu);
+        if (best_nt == 0 || cost < best) {
+            best = cost;
+            best_nt = nt;
+        }
+    }
+    if (best_nt == 1) {
+        const int waves = ntiles >= 512 ? 8 : 16;
+        return SmallMConfig{1, waves, M > 16 ? 1 : 2};
+    }
+    // Two k-tiles per batch only pay where registers allow two resident workgroups:
+    // not with the RMSnorm prologue (146 registers with NT = 2: 20.4 us against 17.9 us).
+    if (best_nt == 2 && M <= 16 && !rms)
+        return SmallMConfig{2, 8, 2};
+    return SmallMConfig{best_nt, 8, 1};
 }
 
 int run_small_m(const GemmArgs &a)

@@ -63,9 +63,10 @@ def test_device_entry_points_validate_before_launch():
     assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 96, 1, 8, None, None, 0, None) == -2   # head size
     assert L.eet_mmha_decode(p, p, None, 0, p, p, p, None, None, 1, 1, 128, 1, 8, None, None, 0, None) == -1     # k without v
     assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 128, 1, 8, p, None, 0, None) == -1  # rotary without k
-    need = L.eet_mmha_decode_workspace(8, 32, 128, 1100)
+    assert L.eet_mmha_decode_workspace(8, 32, 128, 1100) == 0     # one workgroup per (b, h): no partial results
+    need = L.eet_mmha_decode_workspace(1, 8, 128, 1100)           # fewer heads than CUs: the time axis is split
     assert need > 0
-    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 8, 32, 128, 1100, 1153, None, None, 0, None) == -4
+    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 8, 128, 1100, 1153, None, None, 0, None) == -4
     assert L.eet_rope_table(None, 4, 128, None) == -1
     assert L.eet_rmsnorm(p, p, p, 1, 20000, 1e-6, None) == -2
     assert L.eet_qkv_split(p, p, p, p, 1, 4, 1, 128, 1, -1, 6, 8, None) == -1  # rows past the cache end

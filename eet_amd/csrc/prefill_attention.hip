@@ -48,11 +48,12 @@ constexpr int kQT = 2;     // 16-query tiles per wavefront
 __device__ __forceinline__ int vt_swizzle(int d) { return (d & 15) ^ ((d >> 3) & 15); }
 
 template <int DH>
-__global__ __launch_bounds__(kThreads) void prefill_attention_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void prefill_attention_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_cache, const _Float16 *__restrict__ v_cache,
     _Float16 *__restrict__ ctx, const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, int H, int S,
     int T_cap, float scale)
 {
+#if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
     constexpr int DC = DH / 32;            // 32-wide d chunks of the first product
     constexpr int DT = DH / 16;            // 16-row d tiles of the second product
     constexpr int KROW = DH * 2 + 16;      // bytes per K row in LDS
@@ -145,6 +146,12 @@ __global__ __launch_bounds__(kThreads) void prefill_attention_kernel(
         }
     };
 
+    const __amdgpu_buffer_rsrc_t ars = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<_Float16 *>(alibi ? alibi + (size_t)h * S : q), 0, alibi ? (unsigned)S * 2u : 0u, 0x00020000);
+    const bool bias_wide = (S % 4 == 0) && (reinterpret_cast<uintptr_t>(alibi) % 8 == 0);
+    // exponentials are taken as 2^x: log2(e) is folded into the logit scale and the bias
+    constexpr float kLog2e = 1.4426950408889634f;
+    const float scale2 = scale * kLog2e;
     const int k_begin = (padb / kBK) * kBK;
     const int k_end = min(S, q0 + kBQ);  // keys beyond the block's last query are never needed
     if (k_begin < k_end)
@@ -153,15 +160,24 @@ __global__ __launch_bounds__(kThreads) void prefill_attention_kernel(
         __syncthreads();  // previous chunk fully consumed
         store_chunk();
         __syncthreads();
-        // ALiBi terms of this chunk's keys, requested before the prefetch below: loads return in
-        // order, so asking for them later would mean waiting for the whole next chunk as well
-        float bias[4][4];
+        // ALiBi terms of this chunk's keys (keys kc0 + 16*kt + 4g .. +3 are 8 contiguous bytes; reads
+        // past the table return zero, those keys are masked anyway), requested before the prefetch
+        // below: loads return in order, so asking for them later would mean waiting for the whole
+        // next chunk as well
+        half4 bias4[4];
+        if (bias_wide) {
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+            for (int kt = 0; kt < 4; ++kt)
+                bias4[kt] = __builtin_bit_cast(
+                    half4, __builtin_amdgcn_raw_buffer_load_b64(ars, (unsigned)((kc0 + 16 * kt + 4 * g) * 2), 0, 0));
+        } else {  // a head's row of the table is not 8-byte aligned (S % 4 != 0): element loads
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                bias[kt][r] = (alibi != nullptr) ? (float)alibi[(size_t)h * S + min(kc0 + 16 * kt + 4 * g + r, S - 1)]
-                                                 : 0.f;
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    bias4[kt][r] = __builtin_bit_cast(
+                        _Float16, __builtin_amdgcn_raw_buffer_load_b16(ars, (unsigned)((kc0 + 16 * kt + 4 * g + r) * 2), 0, 0));
+        }
         __builtin_amdgcn_sched_barrier(0);
         if (kc0 + kBK < k_end)
             load_chunk(kc0 + kBK);
@@ -194,13 +210,17 @@ __global__ __launch_bounds__(kThreads) void prefill_attention_kernel(
         for (int qt = 0; qt < kQT; ++qt) {
             const int qi = wq0 + 16 * qt + j;
             float cmax = -INFINITY;
+            // only chunks that touch the diagonal or the padded prefix need the mask
+            const bool need_mask = (kc0 + kBK - 1 > wq0) || (kc0 < padb);
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const int key = kc0 + 16 * kt + 4 * g + r;
-                    float s = sacc[qt][kt][r] * scale + bias[kt][r];
-                    s = (key > qi || key < padb) ? -INFINITY : s;
+                    float s = sacc[qt][kt][r] * scale2 + (float)bias4[kt][r] * kLog2e;
+                    if (need_mask) {
+                        const int key = kc0 + 16 * kt + 4 * g + r;
+                        s = (key > qi || key < padb) ? -INFINITY : s;
+                    }
                     sacc[qt][kt][r] = s;
                     cmax = fmaxf(cmax, s);
                 }
@@ -208,14 +228,14 @@ __global__ __launch_bounds__(kThreads) void prefill_attention_kernel(
             cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
             const float m_new = fmaxf(m_run[qt], cmax);
             const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-            const float corr = __expf(m_run[qt] - m_safe);  // 0 while nothing has been seen
+            const float corr = __builtin_amdgcn_exp2f(m_run[qt] - m_safe);  // 0 while nothing has been seen
             float psum = 0.f;
             float p[4][4];
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    p[kt][r] = __expf(sacc[qt][kt][r] - m_safe);
+                    p[kt][r] = __builtin_amdgcn_exp2f(sacc[qt][kt][r] - m_safe);
                     psum += p[kt][r];
                 }
             l_run[qt] = l_run[qt] * corr + psum;  // per-lane share; lanes of a query are summed at the end
@@ -274,6 +294,7 @@ __global__ __launch_bounds__(kThreads) void prefill_attention_kernel(
             *reinterpret_cast<half4 *>(dst + 16 * dt + 4 * g) = o;
         }
     }
+#endif
 }
 
 template <int DH>

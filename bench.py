@@ -290,8 +290,9 @@ def main():
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
-              "(the path has no collectives; see DESIGN.md for how it would shard).", file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported (the path has no "
+              "collectives: a linear would shard by output channels, or by input features with one all-reduce).",
+              file=sys.stderr)
         sys.exit(2)
 
     import torch

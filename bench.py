@@ -337,7 +337,7 @@ def main():
                      "avg_launch_us": round(per_launch_us, 3),
                      "algorithmic_bytes_per_launch": round(step_bytes / launches),
                      # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE (x2.000, calibrated on a
-                     # 1 GiB copy) + WRITE_SIZE (x1.000) at the default workload; see profiles/
+                     # 1 GiB copy) + WRITE_SIZE (x1.000) at the default workload (measured once, not per run)
                      "traffic": 51.73e6 if (M == 8 and args.layers == 32) else None},
         "host_wall_ms_per_step": round(wall * 1e3, 4),
     }

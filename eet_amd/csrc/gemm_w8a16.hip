@@ -443,9 +443,13 @@ static int run_gemm(const GemmArgs &a)
 {
     if (a.M <= 32)
         return run_small_m(a);
-    if (a.M <= 128) {
-        // Too few 128 x 256 tiles to occupy the chip: run the small-M kernel over
-        // 32-row slabs instead (the weights are re-read per slab, from L2 / Infinity Cache).
+    // 33 <= M <= 64 with few channels: the 32 x 128 MFMA tiles would number under ~150 and each
+    // would walk the whole k range alone (19 us at N = 4096, K = 4096 whatever M is), so the
+    // small-M kernel runs over 32-row slabs instead (12-15 us; the weights are re-read per slab,
+    // from L2 / Infinity Cache).  Measured crossover: slabs win for M <= 64 at N = 4096, the
+    // tiles from M = 96 on and for N >= 12288 at any M.
+    const int tile_wgs = ((a.M + 31) / 32) * ((a.N + 127) / 128);
+    if (a.M <= 64 && tile_wgs < 150) {
         const int n_out = (a.epi == kEpiSwiglu) ? a.N / 2 : a.N;
         for (int m0 = 0; m0 < a.M; m0 += 32) {
             GemmArgs s = a;

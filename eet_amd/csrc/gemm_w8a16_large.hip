@@ -357,8 +357,7 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
         // (2 x (kPerWave DMA + TN weight loads)), then the barrier.
         // (A plain __syncthreads() would drain every outstanding load here: its
         // release fence waits for all DMA writes, including the ones just issued.)
-        static_assert(2 * (S::kPerWave + TN) == 16, "the wait count below is written out as a literal");
-        asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * (S::kPerWave + TN)) : "memory");
     };
 
     // prologue: tiles 0..2 into stages 0..2, weights of tiles 0 and 1
@@ -470,8 +469,8 @@ struct LargeMConfig {
 //   128 x 320 (8 wavefronts) wins when it divides the problem into whole rounds of
 //     256 workgroups where 128 x 256 leaves a CU with two tiles against one elsewhere
 //     (M = 2048, N = 5120: 256 tiles instead of 320);
-//   64 x 128 and 32 x 128 keep the chip occupied for M in the hundreds, where the
-//     k-loop latency of the few large tiles would dominate.
+//   64 x 256, 64 x 128 and 32 x 128 (DMA kernel) keep the chip occupied for M in the
+//     hundreds, where the k-loop latency of the few large tiles would dominate.
 LargeMConfig pick_large_m(int M, int N, int epi)
 {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
@@ -485,9 +484,11 @@ LargeMConfig pick_large_m(int M, int N, int epi)
         }
         return LargeMConfig{0, 4, 8, 4};
     }
+    if (wgs(64, 256) >= 600)
+        return LargeMConfig{0, 4, 4, 4};
     if (wgs(64, 128) >= 300)
-        return LargeMConfig{1, 4, 4, 2};
-    return LargeMConfig{1, 4, 2, 2};
+        return LargeMConfig{0, 4, 4, 2};
+    return LargeMConfig{0, 4, 2, 2};
 }
 
 }  // namespace
@@ -504,16 +505,18 @@ int eet::run_large_m(const GemmArgs &a)
         if (sscanf(env, "%d,%d,%d,%d", &e.wmw, &e.wnw, &e.tm, &e.tn) == 4 && (a.epi != kEpiSwiglu || e.tn % 2 == 0))
             c = e;
     }
-    if (c.wmw == 0 && c.wnw == 4 && c.tm == 8 && c.tn == 4)
-        return launch_large_m_dma<4, 8, 4>(a);
-#define EET_LM_CASE(A_, B_, C_, D_)                                      \
-    if (c.wmw == A_ && c.wnw == B_ && c.tm == C_ && c.tn == D_)         \
-        return launch_large_m<A_, B_, C_, D_>(a);
-    EET_LM_CASE(1, 4, 8, 4)
-    EET_LM_CASE(2, 4, 4, 5)
-    EET_LM_CASE(1, 4, 4, 2)
-    EET_LM_CASE(1, 4, 2, 2)
-#undef EET_LM_CASE
+    if (c.wmw == 0 && c.wnw == 4) {
+        if (c.tm == 8 && c.tn == 4)
+            return launch_large_m_dma<4, 8, 4>(a);
+        if (c.tm == 4 && c.tn == 4)
+            return launch_large_m_dma<4, 4, 4>(a);
+        if (c.tm == 4 && c.tn == 2)
+            return launch_large_m_dma<4, 4, 2>(a);
+        if (c.tm == 2 && c.tn == 2)
+            return launch_large_m_dma<4, 2, 2>(a);
+    }
+    if (c.wmw == 2 && c.wnw == 4 && c.tm == 4 && c.tn == 5)
+        return launch_large_m<2, 4, 4, 5>(a);
     return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no large-M kernel for tile %d,%d,%d,%d", c.wmw, c.wnw,
                      c.tm, c.tn);
 }

@@ -1,4 +1,5 @@
-// Large-M fused dequant-GEMM (M > 128, prefill; fp16-MFMA bound).
+// Large-M fused dequant-GEMM (M > 32 apart from the 32-row-slab case; prefill;
+// fp16-MFMA bound).
 //
 // Replaces the tensor-core side of fastertransformer::gemm_fp16_int_bias_act<uint8_t>
 // (3rdparty/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm_template.h:48-177).
@@ -9,18 +10,21 @@
 // such a kernel on a CU is the LDS port (128 B/clk) against the matrix cores
 // (4 x 1024 flop/clk): a wavefront tile of WM x WN outputs needs (WM + WN) * 2 B
 // of operands per k for 2 * WM * WN flop, so wavefront tiles are made large
-// (128 x 64) and only one operand goes through LDS:
+// (128 x 64 where M allows) and only one operand goes through LDS:
 //   weights      every wavefront reads its own TN packed tiles straight from
 //                global memory into registers -- the packed layout is already
 //                the MFMA operand layout -- and widens them once per k-tile;
-//   activations  the block's rows x 64 slab is loaded row-wise (whole 128-byte
-//                lines), written to LDS in operand order with an XOR swizzle
-//                (conflict-free 16-byte writes and reads) and read by every
-//                wavefront of its row group.
-// Both streams are prefetched one k-tile ahead into registers; LDS is double
-// buffered, one barrier per k-tile.  Workgroups are numbered so that the ones
-// sharing a weight column block run on the same XCD (workgroup i lands on XCD
-// i % 8) and hit its L2.
+//   activations  the block's rows x 64 slab goes to LDS in an XOR-swizzled
+//                layout (conflict-free 16-byte writes and reads) and is read
+//                by every wavefront of its row group.
+// Workgroups are numbered so that the ones sharing a weight column block run
+// on the same XCD (workgroup i lands on XCD i % 8) and hit its L2.
+//
+// Two kernels.  w8a16_large_m_kernel stages the activations through registers,
+// one k-tile ahead, LDS double buffered (used for the 128 x 320 tile of eight
+// wavefronts).  w8a16_large_m_dma_kernel, further down, lets the memory
+// pipeline copy them global -> LDS three k-tiles ahead and is the one that runs
+// for every other tile.
 #include <cstdlib>
 
 #include "gemm_common.h"

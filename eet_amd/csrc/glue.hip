@@ -78,6 +78,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(const _Float16 *_
 // One thread handles 4 adjacent pairs, i.e. two 8-byte pieces of each of q,k,v.
 // ---------------------------------------------------------------------------
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+constexpr int kRopeMaxPairs = 128;  // head sizes up to 256 keep their angles in LDS
 
 __global__ void qkv_split_kernel(const _Float16 *__restrict__ qkv, _Float16 *__restrict__ q_out,
                                  _Float16 *__restrict__ k_cache, _Float16 *__restrict__ v_cache, int S, int H,
@@ -86,6 +87,18 @@ __global__ void qkv_split_kernel(const _Float16 *__restrict__ qkv, _Float16 *__r
     const int s = blockIdx.x, b = blockIdx.y;
     const int half_dh = dh / 2;
     const int per_head = half_dh / 4;  // threads per head
+    // All heads of a row turn by the same dh/2 angles: computed once per workgroup.
+    __shared__ float rot_cos[kRopeMaxPairs], rot_sin[kRopeMaxPairs];
+    const bool table = rope && half_dh <= kRopeMaxPairs;
+    if (table) {
+        const float pos = (float)(time_step >= 0 ? time_step : s);
+        for (int i = threadIdx.x; i < half_dh; i += blockDim.x) {
+            const float ang = pos / powf(10000.0f, (float)(2 * i) / (float)dh);
+            rot_cos[i] = cosf(ang);
+            rot_sin[i] = sinf(ang);
+        }
+        __syncthreads();
+    }
     for (int idx = threadIdx.x; idx < H * per_head; idx += blockDim.x) {
         const int h = idx / per_head, i0 = (idx % per_head) * 4;
         const size_t src = ((size_t)(b * S + s) * 3) * H * dh + (size_t)h * dh + i0;
@@ -99,8 +112,15 @@ __global__ void qkv_split_kernel(const _Float16 *__restrict__ qkv, _Float16 *__r
             const float pos = (float)(time_step >= 0 ? time_step : s);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const float ang = pos / powf(10000.0f, (float)(2 * (i0 + e)) / (float)dh);
-                const float c = cosf(ang), sn = sinf(ang);
+                float c, sn;
+                if (table) {
+                    c = rot_cos[i0 + e];
+                    sn = rot_sin[i0 + e];
+                } else {
+                    const float ang = pos / powf(10000.0f, (float)(2 * (i0 + e)) / (float)dh);
+                    c = cosf(ang);
+                    sn = sinf(ang);
+                }
                 const float a = (float)q1[e], bq = (float)q2[e];
                 q1[e] = (_Float16)(a * c - bq * sn);
                 q2[e] = (_Float16)(bq * c + a * sn);

@@ -4,27 +4,34 @@
 // Replaces the tensor-core side of fastertransformer::gemm_fp16_int_bias_act<uint8_t>
 // (3rdparty/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm_template.h:48-177).
 //
-// A workgroup of WMW x WNW wavefronts owns a block tile of (WMW*TM*16) rows x
-// (WNW*TN*16) channels; each wavefront owns TM x TN tiles of
+// A workgroup of WNW wavefronts side by side owns a block tile of TM*16 rows x
+// WNW*TN*16 channels; each wavefront owns TM x TN tiles of
 // v_mfma_f32_16x16x32_f16 (TM*TN*4 fp32 accumulator registers).  What bounds
 // such a kernel on a CU is the LDS port (128 B/clk) against the matrix cores
 // (4 x 1024 flop/clk): a wavefront tile of WM x WN outputs needs (WM + WN) * 2 B
 // of operands per k for 2 * WM * WN flop, so wavefront tiles are made large
 // (128 x 64 where M allows) and only one operand goes through LDS:
 //   weights      every wavefront reads its own TN packed tiles straight from
-//                global memory into registers -- the packed layout is already
-//                the MFMA operand layout -- and widens them once per k-tile;
-//   activations  the block's rows x 64 slab goes to LDS in an XOR-swizzled
-//                layout (conflict-free 16-byte writes and reads) and is read
-//                by every wavefront of its row group.
-// Workgroups are numbered so that the ones sharing a weight column block run
-// on the same XCD (workgroup i lands on XCD i % 8) and hit its L2.
+//                global memory into registers, two k-tiles ahead -- the packed
+//                layout is already the MFMA operand layout -- and widens them
+//                once per k-tile;
+//   activations  the block's rows x 64 slab is copied global -> LDS by the
+//                memory pipeline itself (buffer_load_dwordx4 ... lds: no
+//                staging registers, no ds_write) into a ring of four k-tile
+//                stages, three tiles ahead of the one being multiplied, and
+//                read from there by every wavefront.
+// One wavefront row per workgroup, so that two (or more) workgroups share a CU
+// with independent barriers; a 256 x 256 block of eight wavefronts with one
+// barrier measured 5-10 % slower than two 128 x 256 blocks.  Workgroups are
+// numbered so that the ones sharing a weight column block run on the same XCD
+// (workgroup i lands on XCD i % 8) and hit its L2.
 //
-// Two kernels.  w8a16_large_m_kernel stages the activations through registers,
-// one k-tile ahead, LDS double buffered (used for the 128 x 320 tile of eight
-// wavefronts).  w8a16_large_m_dma_kernel, further down, lets the memory
-// pipeline copy them global -> LDS three k-tiles ahead and is the one that runs
-// for every other tile.
+// A stage holds TM m-tiles of 2 KiB: [row half b][row r (8)][position (8)] x
+// 16 B, where position p of row (b, r) holds piece p ^ ((r >> 1) | (b << 2)) of
+// the row's eight 16-byte pieces.  One DMA instruction fills 1 KiB (8 rows x
+// 128 B, whole cache lines; the XOR only permutes lanes within a line), and the
+// MFMA operand read of lane (g, j) -- piece 2g+h of row j -- hits 16 distinct
+// 16-byte bank groups per 16 lanes.
 #include <cstdlib>
 
 #include "gemm_common.h"
@@ -33,200 +40,6 @@ using namespace eet;
 
 namespace {
 
-template <int WMW, int WNW, int TM, int TN>
-struct LmShape {
-    static constexpr int kThreads = 64 * WMW * WNW;
-    static constexpr int kBM = WMW * TM * 16, kBN = WNW * TN * 16;
-    static constexpr int kPieces = kBM * 8 / kThreads;  // 16-byte activation pieces per thread and k-tile
-    static constexpr int kBufVec = (kBM / 16) * 2 * 64; // u32x4 per LDS buffer: [m-tile][k-half][64 slots]
-    static_assert(kBM * 8 % kThreads == 0, "activation slab must divide evenly over the threads");
-    static_assert(2 * kBufVec * 16 <= 65536, "two activation buffers must fit 64 KiB");
-};
-
-template <int WMW, int WNW, int TM, int TN>
-__global__ __launch_bounds__(64 * WMW * WNW) __attribute__((amdgpu_waves_per_eu(2))) void w8a16_large_m_kernel(
-    const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
-    _Float16 *__restrict__ C, int M, int N, int K, int m_blocks, int n_blocks,
-    const _Float16 *__restrict__ residual, int epi)
-{
-    using S = LmShape<WMW, WNW, TM, TN>;
-    __shared__ u32x4 lds[2][S::kBufVec];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WNW, wn = wave % WNW;
-    const int g = lane >> 4, j = lane & 15;
-    const int ktiles = K >> 6, ntiles = N >> 4;
-
-    // XCD-aware tile order: consecutive workgroups of one XCD walk down the
-    // m-blocks of the same n-block.
-    const int total = m_blocks * n_blocks;
-    const int per_xcd = (total + 7) / 8;
-    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (tile >= total)
-        return;
-    const int n_blk = tile / m_blocks, m_blk = tile % m_blocks;
-    const int m0 = m_blk * S::kBM;
-    const int nt0 = n_blk * (WNW * TN) + wn * TN;
-
-    // A tile index past the end is clamped: its results are never written.
-    const u32x4 *wbase[TN];
-#pragma unroll
-    for (int t = 0; t < TN; ++t)
-        wbase[t] = Wp + (size_t)min(nt0 + t, ntiles - 1) * ktiles * 64 + lane;
-
-    // Activation pieces: rows x 8 pieces of 16 bytes.  Piece p of row r goes to
-    // block (r/16, p%2), slot (p/2)*16 + ((r%16) ^ p): lane (g, j) of k-half h
-    // then finds its operand (piece 2g+h of row j) at slot g*16 + (j ^ (2g+h)).
-    // Rows past M read row M-1; those outputs are never written.
-    const u32x4 *asrc[S::kPieces];
-    int adst[S::kPieces];
-#pragma unroll
-    for (int i = 0; i < S::kPieces; ++i) {
-        const int q = tid + S::kThreads * i, row = q >> 3, p = q & 7;
-        asrc[i] = reinterpret_cast<const u32x4 *>(A + (size_t)min(m0 + row, M - 1) * K) + p;
-        adst[i] = ((row >> 4) * 2 + (p & 1)) * 64 + (p >> 1) * 16 + ((row & 15) ^ p);
-    }
-
-    floatx4 acc[TN][TM];
-#pragma unroll
-    for (int t = 0; t < TN; ++t)
-#pragma unroll
-        for (int mt = 0; mt < TM; ++mt)
-            acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    u32x4 wcur[TN], wnext[TN], areg[S::kPieces];
-#pragma unroll
-    for (int t = 0; t < TN; ++t)
-        wcur[t] = wbase[t][0];
-#pragma unroll
-    for (int i = 0; i < S::kPieces; ++i)
-        areg[i] = asrc[i][0];
-#pragma unroll
-    for (int i = 0; i < S::kPieces; ++i)
-        lds[0][adst[i]] = areg[i];
-    __syncthreads();
-
-    const int rslot0 = wm * TM * 128 + g * 16 + (j ^ (2 * g)), rslot1 = wm * TM * 128 + 64 + g * 16 + (j ^ (2 * g + 1));
-    for (int kt = 0; kt < ktiles; ++kt) {
-        // prefetch the next k-tile (the last iteration re-reads its own tile: no branch around the loads)
-        const int kn = min(kt + 1, ktiles - 1);
-#pragma unroll
-        for (int t = 0; t < TN; ++t)
-            wnext[t] = wbase[t][(size_t)kn * 64];
-#pragma unroll
-        for (int i = 0; i < S::kPieces; ++i)
-            areg[i] = asrc[i][kn * 8];
-        __builtin_amdgcn_sched_barrier(0);
-        half8 w0[TN], w1[TN];
-#pragma unroll
-        for (int t = 0; t < TN; ++t) {
-            w0[t] = widen8(wcur[t].x, wcur[t].y);
-            w1[t] = widen8(wcur[t].z, wcur[t].w);
-        }
-        const u32x4 *buf = lds[kt & 1];
-        // The A operands of m-tile mt+1 are requested before the products of m-tile
-        // mt are issued, into the other register pair (the group barriers below pin
-        // that order; left alone the scheduler reuses one pair and waits on every read).
-        half8 aop[2][2];
-        aop[0][0] = __builtin_bit_cast(half8, buf[rslot0]);
-        aop[0][1] = __builtin_bit_cast(half8, buf[rslot1]);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int mt = 0; mt < TM; ++mt) {
-            if (mt + 1 < TM) {
-                aop[(mt + 1) & 1][0] = __builtin_bit_cast(half8, buf[(mt + 1) * 128 + rslot0]);
-                aop[(mt + 1) & 1][1] = __builtin_bit_cast(half8, buf[(mt + 1) * 128 + rslot1]);
-            }
-#pragma unroll
-            for (int t = 0; t < TN; ++t) {
-                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w0[t], aop[mt & 1][0], acc[t][mt], 0, 0, 0);
-                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w1[t], aop[mt & 1][1], acc[t][mt], 0, 0, 0);
-            }
-        }
-#pragma unroll
-        for (int mt = 0; mt < TM; ++mt) {
-            if (mt + 1 < TM)
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // 2 LDS reads
-            __builtin_amdgcn_sched_group_barrier(0x008, 2 * TN, 0);  // 2*TN MFMA
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < S::kPieces; ++i)
-            lds[(kt + 1) & 1][adst[i]] = areg[i];
-#pragma unroll
-        for (int t = 0; t < TN; ++t)
-            wcur[t] = wnext[t];
-        __syncthreads();
-    }
-
-    // acc[t][mt][r] of lane (g, j): row m0 + 16*(wm*TM + mt) + j, channel 16*(nt0+t) + 4*g + r
-    const int mrow0 = m0 + 16 * wm * TM + j;
-    if (epi == kEpiSwiglu) {
-        if constexpr (TN % 2 == 0) {
-#pragma unroll
-            for (int t = 0; t < TN; t += 2) {
-                if (nt0 + t + 1 >= ntiles)
-                    continue;
-                const half4 sg = *reinterpret_cast<const half4 *>(scale + (nt0 + t) * 16 + 4 * g);
-                const half4 su = *reinterpret_cast<const half4 *>(scale + (nt0 + t + 1) * 16 + 4 * g);
-                const int n = ((nt0 + t) / 2) * 16 + 4 * g;
-#pragma unroll
-                for (int mt = 0; mt < TM; ++mt) {
-                    const int m = mrow0 + 16 * mt;
-                    if (m < M) {
-                        half4 o;
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            // gate and up are rounded to fp16 first, as the separate GEMMs would leave them
-                            const float gate = (float)(_Float16)(acc[t][mt][r] * (float)sg[r]);
-                            const float up = (float)(_Float16)(acc[t + 1][mt][r] * (float)su[r]);
-                            o[r] = (_Float16)(up * gate / (1.0f + __expf(-gate)));
-                        }
-                        *reinterpret_cast<half4 *>(C + (size_t)m * (N / 2) + n) = o;
-                    }
-                }
-            }
-        }
-        return;
-    }
-#pragma unroll
-    for (int t = 0; t < TN; ++t) {
-        if (nt0 + t >= ntiles)
-            continue;
-        const int n = (nt0 + t) * 16 + 4 * g;
-        const half4 sc = *reinterpret_cast<const half4 *>(scale + n);
-#pragma unroll
-        for (int mt = 0; mt < TM; ++mt) {
-            const int m = mrow0 + 16 * mt;
-            if (m < M) {
-                half4 o;
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    o[r] = (_Float16)(acc[t][mt][r] * (float)sc[r]);
-                if (epi == kEpiResidual)
-                    o = o + *reinterpret_cast<const half4 *>(residual + (size_t)m * N + n);  // fp16 add of the rounded product
-                *reinterpret_cast<half4 *>(C + (size_t)m * N + n) = o;
-            }
-        }
-    }
-}
-
-
-// ---------------------------------------------------------------------------
-// Variant with the activations copied global -> LDS by the memory pipeline
-// itself (global_load_lds_dwordx4: no staging registers, no ds_write) into a
-// ring of four k-tile stages, three tiles ahead of the one being multiplied,
-// and the packed weights prefetched two tiles ahead into registers.  One
-// wavefront row (WMW = 1): the block is TM*16 rows x WNW*TN*16 channels, and two
-// such workgroups share a CU with independent barriers.
-//
-// A stage holds TM m-tiles of 2 KiB: [row half b][row r (8)][position (8)] x
-// 16 B, where position p of row (b, r) holds piece p ^ ((r >> 1) | (b << 2)) of
-// the row's eight 16-byte pieces.  One DMA instruction fills 1 KiB (8 rows x
-// 128 B, whole cache lines; the XOR only permutes lanes within a line), and the
-// MFMA operand read of lane (g, j) -- piece 2g+h of row j -- hits 16 distinct
-// 16-byte bank groups per 16 lanes.
-// ---------------------------------------------------------------------------
 constexpr int kDmaStages = 4, kDmaAhead = 3;
 
 __device__ __forceinline__ constexpr int vmcnt_imm(int n)
@@ -246,7 +59,7 @@ struct DmaShape {
 };
 
 template <int WNW, int TM, int TN>
-__global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) void w8a16_large_m_dma_kernel(
+__global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) void w8a16_large_m_kernel(
     const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
     _Float16 *__restrict__ C, int M, int N, int K, int m_blocks, int n_blocks,
     const _Float16 *__restrict__ residual, int epi)
@@ -440,87 +253,74 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
 }
 
 template <int WNW, int TM, int TN>
-int launch_large_m_dma(const GemmArgs &a)
+int launch_large_m(const GemmArgs &a)
 {
     using S = DmaShape<WNW, TM, TN>;
     const int m_blocks = (a.M + S::kBM - 1) / S::kBM, n_blocks = (a.N + S::kBN - 1) / S::kBN;
     const int grid = ((m_blocks * n_blocks + 7) / 8) * 8;
-    hipLaunchKernelGGL((w8a16_large_m_dma_kernel<WNW, TM, TN>), dim3(grid), dim3(S::kThreads), 0, a.st, a.A, a.Wp,
-                       a.scale, a.C, a.M, a.N, a.K, m_blocks, n_blocks, a.residual, a.epi);
-    EET_HIP_CHECK(hipGetLastError());
-    return EET_OK;
-}
-
-template <int WMW, int WNW, int TM, int TN>
-int launch_large_m(const GemmArgs &a)
-{
-    using S = LmShape<WMW, WNW, TM, TN>;
-    const int m_blocks = (a.M + S::kBM - 1) / S::kBM, n_blocks = (a.N + S::kBN - 1) / S::kBN;
-    const int grid = ((m_blocks * n_blocks + 7) / 8) * 8;
-    hipLaunchKernelGGL((w8a16_large_m_kernel<WMW, WNW, TM, TN>), dim3(grid), dim3(S::kThreads), 0, a.st, a.A, a.Wp,
+    hipLaunchKernelGGL((w8a16_large_m_kernel<WNW, TM, TN>), dim3(grid), dim3(S::kThreads), 0, a.st, a.A, a.Wp,
                        a.scale, a.C, a.M, a.N, a.K, m_blocks, n_blocks, a.residual, a.epi);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
 
 struct LargeMConfig {
-    int wmw, wnw, tm, tn;  // wmw = 0: the DMA kernel (one wavefront row)
+    int tm, tn;  // m-tiles and n-tiles of 16 per wavefront; the block is tm*16 rows x 4*tn*16 channels
 };
 
-// Shape -> tile.  Measured on MI355X (M = 129 .. 8192, LLaMA-7B and Baichuan-13B shapes):
-//   128 x 256 (DMA kernel, two workgroups per CU) is the fastest tile once it yields
-//     a few hundred workgroups;
-//   128 x 320 (8 wavefronts) wins when it divides the problem into whole rounds of
-//     256 workgroups where 128 x 256 leaves a CU with two tiles against one elsewhere
-//     (M = 2048, N = 5120: 256 tiles instead of 320);
-//   64 x 256, 64 x 128 and 32 x 128 (DMA kernel) keep the chip occupied for M in the
-//     hundreds, where the k-loop latency of the few large tiles would dominate.
+// Shape -> tile.  Measured on MI355X (M = 33 .. 8192, LLaMA-7B and Baichuan-13B shapes):
+//   128 x 256 (two workgroups per CU) is the fastest tile once it yields a few
+//     hundred workgroups;
+//   64 x 320 wins when it divides the problem into whole rounds of 512 workgroups
+//     where 128 x 256 leaves a CU with two tiles against one elsewhere (M = 2048,
+//     N = 5120: 512 tiles, two per CU, instead of 320);
+//   64 x 256, 64 x 128 and 32 x 128 keep the chip occupied for M in the tens and
+//     hundreds, where the k-loop latency of a few large tiles would dominate.
 LargeMConfig pick_large_m(int M, int N, int epi)
 {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     const int big = wgs(128, 256);
     if (big >= 320) {
-        if (epi != kEpiSwiglu) {  // 128 x 320 holds 5 n-tiles per wavefront: no (gate, up) pairs
+        if (epi != kEpiSwiglu) {  // 5 n-tiles per wavefront: no (gate, up) pairs
+            // time in units of one 128 x 256 tile on a CU of its own; 64 x 320 is 0.625 of that
+            // area and runs at about 0.9 of the large tile's rate
             const double cost_big = 2.0 * ((big + 511) / 512);
-            const double cost_320 = ((wgs(128, 320) + 255) / 256) * (320.0 / 256.0) / 0.9;
+            const double cost_320 = 2.0 * ((wgs(64, 320) + 511) / 512) * 0.625 / 0.9;
             if (cost_320 < cost_big)
-                return LargeMConfig{2, 4, 4, 5};
+                return LargeMConfig{4, 5};
         }
-        return LargeMConfig{0, 4, 8, 4};
+        return LargeMConfig{8, 4};
     }
     if (wgs(64, 256) >= 600)
-        return LargeMConfig{0, 4, 4, 4};
+        return LargeMConfig{4, 4};
     if (wgs(64, 128) >= 300)
-        return LargeMConfig{0, 4, 4, 2};
-    return LargeMConfig{0, 4, 2, 2};
+        return LargeMConfig{4, 2};
+    return LargeMConfig{2, 2};
 }
 
 }  // namespace
 
 int eet::run_large_m(const GemmArgs &a)
 {
-    // the kernels address A rows and the packed weights with 32-bit byte offsets
+    // the kernel addresses A rows and the packed weights with 32-bit byte offsets
     if ((size_t)a.K * a.N >= (1ull << 31) || (size_t)a.K * 2 * 256 >= (1ull << 31))
         return eet::fail(EET_ERR_UNSUPPORTED_SHAPE, "eet_gemm_w8a16: K x N = %d x %d exceeds the 2 GiB weight limit",
                          a.K, a.N);
     LargeMConfig c = pick_large_m(a.M, a.N, a.epi);
-    if (const char *env = std::getenv("EET_GEMM_LARGE_M_TILE")) {  // "wmw,wnw,tm,tn": tuning override
+    if (const char *env = std::getenv("EET_GEMM_LARGE_M_TILE")) {  // "tm,tn": tuning override
         LargeMConfig e = c;
-        if (sscanf(env, "%d,%d,%d,%d", &e.wmw, &e.wnw, &e.tm, &e.tn) == 4 && (a.epi != kEpiSwiglu || e.tn % 2 == 0))
+        if (sscanf(env, "%d,%d", &e.tm, &e.tn) == 2 && (a.epi != kEpiSwiglu || e.tn % 2 == 0))
             c = e;
     }
-    if (c.wmw == 0 && c.wnw == 4) {
-        if (c.tm == 8 && c.tn == 4)
-            return launch_large_m_dma<4, 8, 4>(a);
-        if (c.tm == 4 && c.tn == 4)
-            return launch_large_m_dma<4, 4, 4>(a);
-        if (c.tm == 4 && c.tn == 2)
-            return launch_large_m_dma<4, 4, 2>(a);
-        if (c.tm == 2 && c.tn == 2)
-            return launch_large_m_dma<4, 2, 2>(a);
-    }
-    if (c.wmw == 2 && c.wnw == 4 && c.tm == 4 && c.tn == 5)
-        return launch_large_m<2, 4, 4, 5>(a);
-    return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no large-M kernel for tile %d,%d,%d,%d", c.wmw, c.wnw,
-                     c.tm, c.tn);
+    if (c.tm == 8 && c.tn == 4)
+        return launch_large_m<4, 8, 4>(a);
+    if (c.tm == 4 && c.tn == 5)
+        return launch_large_m<4, 4, 5>(a);
+    if (c.tm == 4 && c.tn == 4)
+        return launch_large_m<4, 4, 4>(a);
+    if (c.tm == 4 && c.tn == 2)
+        return launch_large_m<4, 4, 2>(a);
+    if (c.tm == 2 && c.tn == 2)
+        return launch_large_m<4, 2, 2>(a);
+    return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no large-M kernel for tile %d,%d", c.tm, c.tn);
 }

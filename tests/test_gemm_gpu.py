@@ -96,7 +96,7 @@ def test_large_m_path(gpu):
         assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32), what=f"M={M}")
 
 
-LARGE_M_TILES = ["0,4,8,4", "0,4,4,4", "0,4,4,2", "0,4,2,2", "2,4,4,5"]
+LARGE_M_TILES = ["8,4", "4,5", "4,4", "4,2", "2,2"]   # m-tiles, n-tiles per wavefront
 
 
 @pytest.mark.parametrize("tile", LARGE_M_TILES)
@@ -112,9 +112,9 @@ def test_large_m_tiles(gpu, monkeypatch, tile):
                      what=f"tile {tile} M={M} K={K} N={N}")
 
 
-@pytest.mark.parametrize("M,K,N,tile", [(1024, 256, 12288, "0,4,8,4"), (2048, 256, 5120, "2,4,4,5"),
-                                        (512, 192, 22016, "0,4,4,4"), (512, 256, 8192, "0,4,4,2"),
-                                        (256, 256, 1024, "0,4,2,2"), (100, 320, 12288, "0,4,2,2"),
+@pytest.mark.parametrize("M,K,N,tile", [(1024, 256, 12288, "128x256"), (2048, 256, 5120, "64x320"),
+                                        (512, 192, 22016, "64x256"), (512, 256, 8192, "64x128"),
+                                        (256, 256, 1024, "32x128"), (100, 320, 12288, "32x128"),
                                         (64, 256, 4096, "slabs")])
 def test_large_m_dispatch(gpu, M, K, N, tile):
     """Shapes on which the dispatcher itself picks each tile (named for the record) -- no override."""

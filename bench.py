@@ -91,7 +91,7 @@ def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup):
 
     def one_pass():
         for (a, w, s, c, m, n, k, epi, res) in calls:
-            rc = f(a, w, s, c, m, n, k, epi, res, None, 0.0, sp)
+            rc = f(a, w, s, c, m, n, k, epi, res, None, 0.0, None, 0, sp)
             if rc:
                 raise RuntimeError(lib.eet_last_error().decode())
     for _ in range(warmup):

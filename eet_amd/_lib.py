@@ -22,7 +22,8 @@ SIGNATURES = {
     "eet_preprocess_ref_sm80": (_i, [_vp, _sz, _sz, _vp]),
     "eet_unprocess_ref_sm80": (_i, [_vp, _sz, _sz, _vp]),
     "eet_gemm_w8a16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _vp]),
-    "eet_gemm_w8a16_fused": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _f, _vp]),
+    "eet_gemm_w8a16_workspace": (_sz, [_i, _i, _i, _i]),
+    "eet_gemm_w8a16_fused": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _f, _vp, _sz, _vp]),
     "eet_mmha_decode_workspace": (_sz, [_i, _i, _i, _i]),
     "eet_mmha_decode": (_i, [_vp, _vp, _vp, _l, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
     "eet_rope_table": (_i, [_vp, _i, _i, _vp]),

@@ -50,10 +50,13 @@ struct GemmArgs {
     int epi;
     const _Float16 *rms_gamma;  // non-null: RMSnorm prologue (small-M kernel only)
     float rms_eps;
+    void *ws;  // optional fp32 workspace (split-k partial results)
+    size_t ws_bytes;
     hipStream_t st;
 };
 
-// gemm_w8a16_large.hip: M > 128, fp16-MFMA bound.
+// gemm_w8a16_large.hip: the MFMA-tile kernel for M > 32, and the workspace it can use.
 int run_large_m(const GemmArgs &a);
+size_t large_m_workspace(int M, int N, int K, int epi);
 
 }  // namespace eet

@@ -439,17 +439,26 @@ int run_small_m(const GemmArgs &a)
 
 }  // namespace
 
+// 33 <= M <= 64 with few channels: see run_gemm.
+static bool takes_slabs(int M, int N)
+{
+    const int tile_wgs = ((M + 31) / 32) * ((N + 127) / 128);
+    return M <= 64 && tile_wgs < 150;
+}
+
 static int run_gemm(const GemmArgs &a)
 {
     if (a.M <= 32)
         return run_small_m(a);
-    // 33 <= M <= 64 with few channels: the 32 x 128 MFMA tiles would number under ~150 and each
-    // would walk the whole k range alone (19 us at N = 4096, K = 4096 whatever M is), so the
-    // small-M kernel runs over 32-row slabs instead (12-15 us; the weights are re-read per slab,
-    // from L2 / Infinity Cache).  Measured crossover: slabs win for M <= 64 at N = 4096, the
-    // tiles from M = 96 on and for N >= 12288 at any M.
-    const int tile_wgs = ((a.M + 31) / 32) * ((a.N + 127) / 128);
-    if (a.M <= 64 && tile_wgs < 150) {
+    // 33 <= M <= 64 with few channels and no workspace to split the k range with: the 32 x 128
+    // MFMA tiles would number under ~150 and each would walk the whole k range alone (19 us at
+    // N = 4096, K = 4096 whatever M is), so the small-M kernel runs over 32-row slabs instead
+    // (12-15 us; the weights are re-read per slab, from L2 / Infinity Cache).  With the workspace
+    // the split MFMA launch is faster still (10-11 us; 16 against 24-34 us at K = 11008).
+    const size_t split_bytes = eet::large_m_workspace(a.M, a.N, a.K, a.epi);
+    const bool can_split = split_bytes > 0 && a.ws != nullptr && a.ws_bytes >= split_bytes &&
+                           reinterpret_cast<uintptr_t>(a.ws) % 16 == 0;
+    if (takes_slabs(a.M, a.N) && !can_split && std::getenv("EET_GEMM_LARGE_M_TILE") == nullptr) {
         const int n_out = (a.epi == kEpiSwiglu) ? a.N / 2 : a.N;
         for (int m0 = 0; m0 < a.M; m0 += 32) {
             GemmArgs s = a;
@@ -482,20 +491,25 @@ static int check_gemm_args(const char *fn, const void *A, const void *W, const v
 extern "C" int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *scale, void *C, int M, int N, int K,
                               void *workspace, size_t workspace_bytes, void *stream)
 {
-    (void)workspace;
-    (void)workspace_bytes;
     if (int rc = check_gemm_args("eet_gemm_w8a16", A, Wpacked, scale, C, M, N, K))
         return rc;
     if (M == 0)
         return EET_OK;
     return run_gemm(GemmArgs{static_cast<const _Float16 *>(A), static_cast<const u32x4 *>(Wpacked),
                              static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(C), M, N, K, nullptr,
-                             kEpiNone, nullptr, 0.f, static_cast<hipStream_t>(stream)});
+                             kEpiNone, nullptr, 0.f, workspace, workspace_bytes, static_cast<hipStream_t>(stream)});
+}
+
+extern "C" size_t eet_gemm_w8a16_workspace(int M, int N, int K, int epilogue)
+{
+    if (M <= 32 || N <= 0 || K <= 0 || K % 64 != 0 || N % 16 != 0)
+        return 0;
+    return eet::large_m_workspace(M, N, K, epilogue);
 }
 
 extern "C" int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, void *C, int M, int N,
                                     int K, int epilogue, const void *residual, const void *rms_gamma, float rms_eps,
-                                    void *stream)
+                                    void *workspace, size_t workspace_bytes, void *stream)
 {
     if (int rc = check_gemm_args("eet_gemm_w8a16_fused", A, Wpacked, scale, C, M, N, K))
         return rc;
@@ -516,5 +530,6 @@ extern "C" int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const vo
     return run_gemm(GemmArgs{static_cast<const _Float16 *>(A), static_cast<const u32x4 *>(Wpacked),
                              static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(C), M, N, K,
                              static_cast<const _Float16 *>(residual), epilogue,
-                             static_cast<const _Float16 *>(rms_gamma), rms_eps, static_cast<hipStream_t>(stream)});
+                             static_cast<const _Float16 *>(rms_gamma), rms_eps, workspace, workspace_bytes,
+                             static_cast<hipStream_t>(stream)});
 }

@@ -62,7 +62,7 @@ template <int WNW, int TM, int TN>
 __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) void w8a16_large_m_kernel(
     const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
     _Float16 *__restrict__ C, int M, int N, int K, int m_blocks, int n_blocks,
-    const _Float16 *__restrict__ residual, int epi)
+    const _Float16 *__restrict__ residual, int epi, int ksplit, float *__restrict__ partial)
 {
 #if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
     using S = DmaShape<WNW, TM, TN>;
@@ -74,6 +74,11 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: feeds scalar offsets and M0
     const int g = lane >> 4, j = lane & 15;
     const int ktiles = K >> 6, ntiles = N >> 4;
+    // With ksplit > 1 (grid.y) the workgroup covers k-tiles [kbeg, kbeg + nk) only and
+    // leaves its raw fp32 sums in partial[split][M][N] for the reduce kernel.
+    const int split = blockIdx.y;
+    const int kbeg = (int)((long)split * ktiles / ksplit);
+    const int nk = (int)((long)(split + 1) * ktiles / ksplit) - kbeg;
 
     const int total = m_blocks * n_blocks;
     const int per_xcd = (total + 7) / 8;
@@ -136,7 +141,7 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
     // One k-tile: A from `cur`, raw weights from wb; the DMA for tile kt + 3 goes
     // to `ahead`, the weights of tile kt + 2 replace wb once it is widened.
     auto step = [&](const u32x4 *cur, u32x4 *ahead, u32x4 (&wb)[TN], int kt) {
-        dma_tile(ahead, min(kt + kDmaAhead, ktiles - 1));
+        dma_tile(ahead, kbeg + min(kt + kDmaAhead, nk - 1));
         __builtin_amdgcn_sched_barrier(0);
         half8 w0[TN], w1[TN];
 #pragma unroll
@@ -145,7 +150,7 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
             w1[t] = widen8(wb[t].z, wb[t].w);
         }
         __builtin_amdgcn_sched_barrier(0);
-        load_w(wb, min(kt + 2, ktiles - 1));
+        load_w(wb, kbeg + min(kt + 2, nk - 1));
         half8 aop[2][2];
         aop[0][0] = __builtin_bit_cast(half8, cur[rs0]);
         aop[0][1] = __builtin_bit_cast(half8, cur[rs1]);
@@ -178,30 +183,45 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
     };
 
     // prologue: tiles 0..2 into stages 0..2, weights of tiles 0 and 1
-    load_w(wraw[0], 0);
-    dma_tile(st0, 0);
-    load_w(wraw[1], min(1, ktiles - 1));
-    dma_tile(st1, min(1, ktiles - 1));
-    dma_tile(st2, min(2, ktiles - 1));
+    load_w(wraw[0], kbeg);
+    dma_tile(st0, kbeg);
+    load_w(wraw[1], kbeg + min(1, nk - 1));
+    dma_tile(st1, kbeg + min(1, nk - 1));
+    dma_tile(st2, kbeg + min(2, nk - 1));
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __syncthreads();
 
     int kt = 0;
-    for (; kt + 4 <= ktiles; kt += 4) {
+    for (; kt + 4 <= nk; kt += 4) {
         step(st0, st3, wraw[0], kt);
         step(st1, st0, wraw[1], kt + 1);
         step(st2, st1, wraw[0], kt + 2);
         step(st3, st2, wraw[1], kt + 3);
     }
-    if (kt < ktiles)
+    if (kt < nk)
         step(st0, st3, wraw[0], kt);
-    if (kt + 1 < ktiles)
+    if (kt + 1 < nk)
         step(st1, st0, wraw[1], kt + 1);
-    if (kt + 2 < ktiles)
+    if (kt + 2 < nk)
         step(st2, st1, wraw[0], kt + 2);
 
     // acc[t][mt][r] of lane (g, j): row m0 + 16*mt + j, channel 16*(nt0+t) + 4*g + r
     const int mrow0 = m0 + j;
+    if (ksplit > 1) {
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+            if (nt0 + t >= ntiles)
+                continue;
+#pragma unroll
+            for (int mt = 0; mt < TM; ++mt) {
+                const int m = mrow0 + 16 * mt;
+                if (m < M)
+                    *reinterpret_cast<floatx4 *>(partial + ((size_t)split * M + m) * N + (nt0 + t) * 16 + 4 * g) =
+                        acc[t][mt];
+            }
+        }
+        return;
+    }
     if (epi == kEpiSwiglu) {
         if constexpr (TN % 2 == 0) {
 #pragma unroll
@@ -252,20 +272,72 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
 #endif
 }
 
+// Second pass of a split-k launch: sums the ksplit partial results of 4 adjacent
+// channels of one row, applies the per-channel scale and the epilogue, rounds once
+// (gate and up are rounded to fp16 before SwiGLU, as the single-pass kernel does).
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ partial,
+                                                            const _Float16 *__restrict__ scale,
+                                                            _Float16 *__restrict__ C,
+                                                            const _Float16 *__restrict__ residual, int M, int N,
+                                                            int ksplit, int epi)
+{
+    const int n_out = (epi == kEpiSwiglu) ? N / 2 : N;
+    const int groups = n_out / 4;
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= M * groups)
+        return;
+    const int m = idx / groups, o4 = (idx % groups) * 4;
+    auto sum4 = [&](int n) {
+        floatx4 s = *reinterpret_cast<const floatx4 *>(partial + (size_t)m * N + n);
+        for (int k = 1; k < ksplit; ++k)
+            s += *reinterpret_cast<const floatx4 *>(partial + ((size_t)k * M + m) * N + n);
+        return s;
+    };
+    half4 o;
+    if (epi == kEpiSwiglu) {
+        const int ng = (o4 / 16) * 32 + o4 % 16, nu = ng + 16;  // gate tile 2u, up tile 2u+1
+        const floatx4 sg = sum4(ng), su = sum4(nu);
+        const half4 cg = *reinterpret_cast<const half4 *>(scale + ng), cu = *reinterpret_cast<const half4 *>(scale + nu);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float gate = (float)(_Float16)(sg[r] * (float)cg[r]);
+            const float up = (float)(_Float16)(su[r] * (float)cu[r]);
+            o[r] = (_Float16)(up * gate / (1.0f + __expf(-gate)));
+        }
+    } else {
+        const floatx4 sv = sum4(o4);
+        const half4 sc = *reinterpret_cast<const half4 *>(scale + o4);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            o[r] = (_Float16)(sv[r] * (float)sc[r]);
+        if (epi == kEpiResidual)
+            o = o + *reinterpret_cast<const half4 *>(residual + (size_t)m * N + o4);
+    }
+    *reinterpret_cast<half4 *>(C + (size_t)m * n_out + o4) = o;
+}
+
 template <int WNW, int TM, int TN>
-int launch_large_m(const GemmArgs &a)
+int launch_large_m(const GemmArgs &a, int ksplit)
 {
     using S = DmaShape<WNW, TM, TN>;
     const int m_blocks = (a.M + S::kBM - 1) / S::kBM, n_blocks = (a.N + S::kBN - 1) / S::kBN;
     const int grid = ((m_blocks * n_blocks + 7) / 8) * 8;
-    hipLaunchKernelGGL((w8a16_large_m_kernel<WNW, TM, TN>), dim3(grid), dim3(S::kThreads), 0, a.st, a.A, a.Wp,
-                       a.scale, a.C, a.M, a.N, a.K, m_blocks, n_blocks, a.residual, a.epi);
+    float *partial = ksplit > 1 ? static_cast<float *>(a.ws) : nullptr;
+    hipLaunchKernelGGL((w8a16_large_m_kernel<WNW, TM, TN>), dim3(grid, ksplit), dim3(S::kThreads), 0, a.st, a.A, a.Wp,
+                       a.scale, a.C, a.M, a.N, a.K, m_blocks, n_blocks, a.residual, a.epi, ksplit, partial);
     EET_HIP_CHECK(hipGetLastError());
+    if (ksplit > 1) {
+        const int items = a.M * ((a.epi == kEpiSwiglu ? a.N / 2 : a.N) / 4);
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((items + 255) / 256), dim3(256), 0, a.st, partial, a.scale, a.C,
+                           a.residual, a.M, a.N, ksplit, a.epi);
+        EET_HIP_CHECK(hipGetLastError());
+    }
     return EET_OK;
 }
 
 struct LargeMConfig {
     int tm, tn;  // m-tiles and n-tiles of 16 per wavefront; the block is tm*16 rows x 4*tn*16 channels
+    int ksplit;  // > 1: that many workgroups share a tile's k range (needs the fp32 workspace)
 };
 
 // Shape -> tile.  Measured on MI355X (M = 33 .. 8192, LLaMA-7B and Baichuan-13B shapes):
@@ -276,7 +348,30 @@ struct LargeMConfig {
 //     N = 5120: 512 tiles, two per CU, instead of 320);
 //   64 x 256, 64 x 128 and 32 x 128 keep the chip occupied for M in the tens and
 //     hundreds, where the k-loop latency of a few large tiles would dominate.
-LargeMConfig pick_large_m(int M, int N, int epi)
+// Estimated time (us) of tile (tm, tn) with the k range split ks ways, for launches
+// too small to fill the chip.  Fitted to MI355X measurements (M = 40 .. 512, LLaMA-7B
+// shapes, within ~10 %): a workgroup alone on its CU needs `lat` us per k-tile
+// (load -> widen -> MFMA latency chain), co-resident workgroups share the CU's
+// L2 bandwidth at `thr` us per k-tile each; a split launch pays a second kernel
+// (~2 us) that reads what the first wrote (ks * M * N fp32, ~4 TB/s effective).
+struct SplitTile {
+    int tm, tn;
+    double lat, thr;
+};
+constexpr SplitTile kSplitTiles[2] = {{2, 2, 0.26, 0.14}, {4, 2, 0.33, 0.23}};
+
+double split_cost_us(int M, int N, int K, const SplitTile &t, int ks)
+{
+    const int wgs = ((M + t.tm * 16 - 1) / (t.tm * 16)) * ((N + t.tn * 64 - 1) / (t.tn * 64)) * ks;
+    const double load = wgs <= 512 ? (double)((wgs + 255) / 256) : wgs / 256.0;
+    const double per_tile = t.lat > t.thr * load ? t.lat : t.thr * load;
+    double us = 2.5 + (K / 64.0 / ks) * per_tile;
+    if (ks > 1)
+        us += 2.0 + (double)ks * M * N * 8.0 / 4e6;
+    return us;
+}
+
+LargeMConfig pick_large_m(int M, int N, int K, int epi, bool may_split)
 {
     auto wgs = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     const int big = wgs(128, 256);
@@ -287,18 +382,38 @@ LargeMConfig pick_large_m(int M, int N, int epi)
             const double cost_big = 2.0 * ((big + 511) / 512);
             const double cost_320 = 2.0 * ((wgs(64, 320) + 511) / 512) * 0.625 / 0.9;
             if (cost_320 < cost_big)
-                return LargeMConfig{4, 5};
+                return LargeMConfig{4, 5, 1};
         }
-        return LargeMConfig{8, 4};
+        return LargeMConfig{8, 4, 1};
     }
     if (wgs(64, 256) >= 600)
-        return LargeMConfig{4, 4};
-    if (wgs(64, 128) >= 300)
-        return LargeMConfig{4, 2};
-    return LargeMConfig{2, 2};
+        return LargeMConfig{4, 4, 1};
+    // Fewer tiles than fill the chip twice: 32 x 128 or 64 x 128, and the k range of
+    // a tile may be shared by up to 8 workgroups (at least 8 k-tiles each) whose fp32
+    // partial sums a small second kernel adds.
+    const int ktiles = K / 64;
+    LargeMConfig best{2, 2, 1};
+    double best_us = 1e30;
+    for (const SplitTile &t : kSplitTiles)
+        for (int ks = 1; ks <= (may_split ? 8 : 1); ++ks) {
+            if (ks > 1 && ktiles / ks < 8)
+                break;
+            const double us = split_cost_us(M, N, K, t, ks);
+            if (us < best_us) {
+                best_us = us;
+                best = LargeMConfig{t.tm, t.tn, ks};
+            }
+        }
+    return best;
 }
 
 }  // namespace
+
+size_t eet::large_m_workspace(int M, int N, int K, int epi)
+{
+    const LargeMConfig c = pick_large_m(M, N, K, epi, true);
+    return c.ksplit > 1 ? (size_t)c.ksplit * M * N * sizeof(float) : 0;
+}
 
 int eet::run_large_m(const GemmArgs &a)
 {
@@ -306,21 +421,36 @@ int eet::run_large_m(const GemmArgs &a)
     if ((size_t)a.K * a.N >= (1ull << 31) || (size_t)a.K * 2 * 256 >= (1ull << 31))
         return eet::fail(EET_ERR_UNSUPPORTED_SHAPE, "eet_gemm_w8a16: K x N = %d x %d exceeds the 2 GiB weight limit",
                          a.K, a.N);
-    LargeMConfig c = pick_large_m(a.M, a.N, a.epi);
-    if (const char *env = std::getenv("EET_GEMM_LARGE_M_TILE")) {  // "tm,tn": tuning override
+    // the split needs room for ksplit x M x N fp32; without it the best single-pass tile
+    auto fits = [&](int ks) {
+        return ks <= 1 || (a.ws != nullptr && reinterpret_cast<uintptr_t>(a.ws) % 16 == 0 &&
+                           a.ws_bytes >= (size_t)ks * a.M * a.N * sizeof(float));
+    };
+    LargeMConfig c = pick_large_m(a.M, a.N, a.K, a.epi, true);
+    if (!fits(c.ksplit))
+        c = pick_large_m(a.M, a.N, a.K, a.epi, false);
+    if (const char *env = std::getenv("EET_GEMM_LARGE_M_TILE")) {  // "tm,tn[,ksplit]": tuning override
         LargeMConfig e = c;
-        if (sscanf(env, "%d,%d", &e.tm, &e.tn) == 2 && (a.epi != kEpiSwiglu || e.tn % 2 == 0))
+        const int got = sscanf(env, "%d,%d,%d", &e.tm, &e.tn, &e.ksplit);
+        if (got >= 2 && (a.epi != kEpiSwiglu || e.tn % 2 == 0)) {
+            if (got == 2)
+                e.ksplit = 1;
             c = e;
+        }
+        if (!fits(c.ksplit))
+            c.ksplit = 1;
     }
+    if (c.ksplit < 1 || c.ksplit > a.K / 64)
+        c.ksplit = 1;
     if (c.tm == 8 && c.tn == 4)
-        return launch_large_m<4, 8, 4>(a);
+        return launch_large_m<4, 8, 4>(a, c.ksplit);
     if (c.tm == 4 && c.tn == 5)
-        return launch_large_m<4, 4, 5>(a);
+        return launch_large_m<4, 4, 5>(a, c.ksplit);
     if (c.tm == 4 && c.tn == 4)
-        return launch_large_m<4, 4, 4>(a);
+        return launch_large_m<4, 4, 4>(a, c.ksplit);
     if (c.tm == 4 && c.tn == 2)
-        return launch_large_m<4, 4, 2>(a);
+        return launch_large_m<4, 4, 2>(a, c.ksplit);
     if (c.tm == 2 && c.tn == 2)
-        return launch_large_m<4, 2, 2>(a);
+        return launch_large_m<4, 2, 2>(a, c.ksplit);
     return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no large-M kernel for tile %d,%d", c.tm, c.tn);
 }

@@ -120,9 +120,16 @@ RMS_FUSE_MAX_M = 32     # the RMSnorm prologue exists in the small-M kernel only
 
 
 def _gemm(a, w, scale, out, M, N, K, epilogue=EPI_NONE, residual=None, rms_gamma=None, rms_eps=0.0):
-    check(lib().eet_gemm_w8a16_fused(a.data_ptr(), w.data_ptr(), scale.data_ptr(), out.data_ptr(), M, N, K,
-                                     epilogue, residual.data_ptr() if residual is not None else None,
-                                     rms_gamma.data_ptr() if rms_gamma is not None else None, rms_eps, _stream()),
+    L = lib()
+    ws, ws_bytes = None, 0
+    if M > RMS_FUSE_MAX_M:    # a launch with few tiles may split its k range: fp32 partial sums
+        ws_bytes = L.eet_gemm_w8a16_workspace(M, N, K, epilogue)
+        if ws_bytes:
+            ws = workspaces.get("gemm_split_k", ws_bytes // 4, torch.float32, a.device).data_ptr()
+    check(L.eet_gemm_w8a16_fused(a.data_ptr(), w.data_ptr(), scale.data_ptr(), out.data_ptr(), M, N, K,
+                                 epilogue, residual.data_ptr() if residual is not None else None,
+                                 rms_gamma.data_ptr() if rms_gamma is not None else None, rms_eps, ws, ws_bytes,
+                                 _stream()),
           "eet_gemm_w8a16_fused")
 
 

@@ -84,7 +84,12 @@ int eet_unprocess_ref_sm80(const int8_t *processed, size_t K, size_t N, int8_t *
 /* C[M][N] (half) = A[M][K] (half) . (int8 W[K][N] * scale[N] (half)), fp32
  * accumulation, one rounding to half.  Wpacked comes from eet_pack_gfx950.
  * M <= 32 takes the HBM-streaming small-M kernel, larger M the LDS-staged MFMA
- * kernel.  No workspace is needed (NULL / 0 accepted).
+ * kernel.  The workspace is optional (NULL / 0 accepted): with
+ * eet_gemm_w8a16_workspace(M, N, K, epilogue) bytes of 16-byte aligned device
+ * memory the library may split the k range of a launch that has too few tiles to
+ * fill the chip (M in the tens to hundreds) and add the parts in a second small
+ * kernel -- the reference's split-k workspace, which its callers never pass
+ * (fpA_intB_gemm_template.h:443-495, cutlass_heuristic.cc:80-84).
  * Replaces fastertransformer::gemm_fp16_int_bias_act<uint8_t>
  * (3rdparty/cutlass_kernels/fpA_intB_gemm.cu:35-62) as called with
  * bias = nullptr and no activation from csrc/op/llama_mmha.cpp:313-337,
@@ -92,6 +97,7 @@ int eet_unprocess_ref_sm80(const int8_t *processed, size_t K, size_t N, int8_t *
 int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *scale, void *C,
                    int M, int N, int K, void *workspace, size_t workspace_bytes,
                    void *stream);
+size_t eet_gemm_w8a16_workspace(int M, int N, int K, int epilogue);
 
 /* The same GEMM with a fused epilogue.
  *   EET_EPILOGUE_NONE      C[M][N] as above.
@@ -110,11 +116,13 @@ int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *scale, void *
  * GEMM -- the RMSnorm + GEMM pairs at csrc/op/llama_mmha.cpp:222-227 and
  * csrc/op/gated_ffn_int8.cpp:112-116 in one launch.  The kernel multiplies
  * x * gamma in fp16 on the way in, accumulates sum(x^2) per row, and applies
- * rsqrt(mean + eps) to the fp32 accumulator. */
+ * rsqrt(mean + eps) to the fp32 accumulator.
+ * workspace / workspace_bytes as for eet_gemm_w8a16 (optional). */
 enum { EET_EPILOGUE_NONE = 0, EET_EPILOGUE_RESIDUAL = 1, EET_EPILOGUE_SWIGLU = 2 };
 int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, void *C,
                          int M, int N, int K, int epilogue, const void *residual,
-                         const void *rms_gamma, float rms_eps, void *stream);
+                         const void *rms_gamma, float rms_eps, void *workspace,
+                         size_t workspace_bytes, void *stream);
 
 /* Masked multi-head decode attention for one new token per sequence.
  *   q, k, v   [B][H][dh] half; with qkv_stride != 0 they are rows of a fused

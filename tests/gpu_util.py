@@ -22,10 +22,33 @@ def assert_close(got, want, rtol=RTOL, atol=ATOL, what=""):
     assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.size} outside tolerance, max err {err.max():.5f}"
 
 
-def gemm(a, wp, s, M, N, K):
+def gemm_workspace(M, N, K, epi, device, min_bytes=0):
+    """(pointer, bytes) of the optional split-k workspace the library asks for
+    (None, 0 when it asks for none); min_bytes forces a larger one for tests
+    that override the split."""
+    need = max(lib().eet_gemm_w8a16_workspace(M, N, K, epi), min_bytes)
+    if not need:
+        return None, 0, None
+    buf = torch.empty(need // 4, dtype=torch.float32, device=device)
+    return buf.data_ptr(), need, buf
+
+
+def gemm(a, wp, s, M, N, K, ws_min_bytes=0):
     c = torch.empty(M, N, dtype=torch.float16, device=a.device)
-    check(lib().eet_gemm_w8a16(a.data_ptr(), wp.data_ptr(), s.data_ptr(), c.data_ptr(), M, N, K, None, 0, stream()),
-          "eet_gemm_w8a16")
+    ws, ws_bytes, keep = gemm_workspace(M, N, K, 0, a.device, ws_min_bytes)
+    check(lib().eet_gemm_w8a16(a.data_ptr(), wp.data_ptr(), s.data_ptr(), c.data_ptr(), M, N, K, ws, ws_bytes,
+                               stream()), "eet_gemm_w8a16")
+    return c
+
+
+def gemm_fused(a, wp, s, M, N, K, epi, residual=None, gamma=None, eps=0.0, ws_min_bytes=0, use_ws=True):
+    n_out = N // 2 if epi == 2 else N
+    c = torch.empty(M, n_out, dtype=torch.float16, device=a.device)
+    ws, ws_bytes, keep = gemm_workspace(M, N, K, epi, a.device, ws_min_bytes) if use_ws else (None, 0, None)
+    check(lib().eet_gemm_w8a16_fused(a.data_ptr(), wp.data_ptr(), s.data_ptr(), c.data_ptr(), M, N, K, epi,
+                                     residual.data_ptr() if residual is not None else None,
+                                     gamma.data_ptr() if gamma is not None else None, eps, ws, ws_bytes, stream()),
+          "eet_gemm_w8a16_fused")
     return c
 
 

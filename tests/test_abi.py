@@ -59,6 +59,12 @@ def test_device_entry_points_validate_before_launch():
     assert L.eet_gemm_w8a16(p, p, p, p, 1, 24, 64, None, 0, None) == -2       # N % 16
     assert b"K % 64" in L.eet_last_error()
     assert L.eet_gemm_w8a16(p, p, p, p, 0, 16, 64, None, 0, None) == 0        # empty batch: nothing to do
+    # split-k workspace: none for the small-M kernel or once the tiles fill the chip, ksplit x M x N fp32 between
+    assert L.eet_gemm_w8a16_workspace(32, 4096, 4096, 0) == 0
+    assert L.eet_gemm_w8a16_workspace(2048, 4096, 4096, 0) == 0
+    need = L.eet_gemm_w8a16_workspace(64, 4096, 11008, 0)
+    assert need >= 2 * 64 * 4096 * 4 and need % (64 * 4096 * 4) == 0
+    assert L.eet_gemm_w8a16_workspace(64, 4100, 11008, 0) == 0                # not a shape the GEMM accepts
     assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 128, 9, 8, None, None, 0, None) == -1  # step > cap
     assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 96, 1, 8, None, None, 0, None) == -2   # head size
     assert L.eet_mmha_decode(p, p, None, 0, p, p, p, None, None, 1, 1, 128, 1, 8, None, None, 0, None) == -1     # k without v
@@ -119,8 +125,8 @@ def test_fused_argument_errors():
     buf = np.zeros(4096, np.uint8)
     p = buf.ctypes.data
     L = lib()
-    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 7, None, None, 0.0, None) == -1          # unknown epilogue
-    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 1, None, None, 0.0, None) == -1          # residual missing
-    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 0, p, None, 0.0, None) == -1             # residual without the epilogue
-    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 48, 64, 2, None, None, 0.0, None) == -2          # odd tile count
-    assert L.eet_gemm_w8a16_fused(p, p, p, p, 64, 32, 64, 0, None, p, 1e-6, None) == -2       # RMSnorm prologue, M > 32
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 7, None, None, 0.0, None, 0, None) == -1          # unknown epilogue
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 1, None, None, 0.0, None, 0, None) == -1          # residual missing
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 0, p, None, 0.0, None, 0, None) == -1             # residual without the epilogue
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 48, 64, 2, None, None, 0.0, None, 0, None) == -2          # odd tile count
+    assert L.eet_gemm_w8a16_fused(p, p, p, p, 64, 32, 64, 0, None, p, 1e-6, None, 0, None) == -2       # RMSnorm prologue, M > 32

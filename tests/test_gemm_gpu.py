@@ -144,15 +144,9 @@ def test_full_size_linearity(gpu):
     assert ((c2 - ca * 2).abs() <= 2.0 ** -24).all()
 
 
-def fused(a, wp, s, M, N, K, epi, residual=None, gamma=None, eps=0.0):
-    from eet_amd._lib import check, lib
-    from gpu_util import stream
-    n_out = N // 2 if epi == 2 else N
-    c = torch.empty(M, n_out, dtype=torch.float16, device=a.device)
-    check(lib().eet_gemm_w8a16_fused(a.data_ptr(), wp.data_ptr(), s.data_ptr(), c.data_ptr(), M, N, K, epi,
-                                     residual.data_ptr() if residual is not None else None,
-                                     gamma.data_ptr() if gamma is not None else None, eps, stream()))
-    return c
+def fused(a, wp, s, M, N, K, epi, residual=None, gamma=None, eps=0.0, **kw):
+    from gpu_util import gemm_fused
+    return gemm_fused(a, wp, s, M, N, K, epi, residual, gamma, eps, **kw)
 
 
 @pytest.mark.parametrize("M", [1, 8, 13, 32, 70, 300])
@@ -210,6 +204,55 @@ def test_large_m_tile_epilogues(gpu, monkeypatch, tile):
     want = O.swiglu(O.dequant_matmul(x.numpy(), ug.numpy(), sg.numpy()),
                     O.dequant_matmul(x.numpy(), uu.numpy(), su.numpy()))
     assert_close(got, want, rtol=1e-2, atol=1e-3)
+
+
+SPLIT_K = ["2,2,2", "2,2,3", "2,2,8", "4,2,4", "4,4,2", "8,4,5"]   # m-tiles, n-tiles, parts of the k range
+
+
+@pytest.mark.parametrize("cfg", SPLIT_K)
+@pytest.mark.parametrize("M,K,N", [(70, 1216, 400), (33, 4096, 1024), (161, 640, 528)])
+def test_split_k(gpu, monkeypatch, cfg, M, K, N):
+    """Every tile with its k range shared by several workgroups (uneven shares, ragged rows and channels,
+    one k-tile per part at K = 640 with 8 parts) + the second kernel that adds the fp32 parts, for all three
+    epilogues, against the fp32 oracle; without the workspace the same call runs in a single pass."""
+    from eet_amd.ops import interleave_gate_up
+    monkeypatch.setenv("EET_GEMM_LARGE_M_TILE", cfg)
+    ws = 8 * M * max(N, 1024) * 4
+    x, u, p, s = make(M, K, N, 11)
+    res = torch.randn(M, N, generator=torch.Generator().manual_seed(M)).half()
+    xd, pd, sd, rd = x.to(gpu), p.to(gpu), s.to(gpu), res.to(gpu)
+    ref = O.dequant_matmul(x.numpy(), u.numpy(), s.numpy())
+    got = gemm(xd, pd, sd, M, N, K, ws_min_bytes=ws).cpu()
+    assert_close(got.numpy(), ref, rtol=1e-2, atol=1e-3)
+    got_r = fused(xd, pd, sd, M, N, K, 1, rd, ws_min_bytes=ws).cpu()
+    assert torch.equal(got_r, got + res)
+    single = fused(xd, pd, sd, M, N, K, 0, use_ws=False).cpu()     # no workspace: one pass, same tile
+    assert_close(single.numpy(), ref, rtol=1e-2, atol=1e-3)
+    F = 272
+    g = torch.Generator().manual_seed(F)
+    wg = (torch.randn(K, F, generator=g) * 0.02).half()
+    wu = (torch.randn(K, F, generator=g) * 0.02).half()
+    ug, pg, sg = eet_amd.quant_weights(wg, torch.int8, True)
+    uu, pu, su = eet_amd.quant_weights(wu, torch.int8, True)
+    w01, s01 = interleave_gate_up(pg, sg, pu, su)
+    got = fused(xd, w01.to(gpu), s01.to(gpu), M, 2 * F, K, 2, ws_min_bytes=ws).cpu().numpy()
+    want = O.swiglu(O.dequant_matmul(x.numpy(), ug.numpy(), sg.numpy()),
+                    O.dequant_matmul(x.numpy(), uu.numpy(), su.numpy()))
+    assert_close(got, want, rtol=1e-2, atol=1e-3)
+
+
+@pytest.mark.parametrize("M,K,N", [(40, 4096, 4096), (64, 11008, 4096), (96, 4096, 4096), (256, 11008, 4096),
+                                   (48, 4096, 12288)])
+def test_split_k_dispatch(gpu, M, K, N):
+    """Shapes for which the library asks for a split-k workspace: the result with it (MFMA tiles, k range
+    split) and without it (32-row slabs of the small-M kernel / single-pass tiles) both match the oracle."""
+    from eet_amd._lib import lib
+    assert lib().eet_gemm_w8a16_workspace(M, N, K, 0) > 0
+    x, u, p, s = make(M, K, N, 13)
+    xd, pd, sd = x.to(gpu), p.to(gpu), s.to(gpu)
+    ref = O.dequant_matmul(x.numpy(), u.numpy(), s.numpy())
+    assert_close(fused(xd, pd, sd, M, N, K, 0).cpu().numpy(), ref, rtol=1e-2, atol=1e-3)
+    assert_close(fused(xd, pd, sd, M, N, K, 0, use_ws=False).cpu().numpy(), ref, rtol=1e-2, atol=1e-3)
 
 
 @pytest.mark.parametrize("M,K,N,epi", [(1, 256, 64, 0), (8, 4096, 12288, 0), (8, 4096, 22016, 2), (16, 1024, 176, 0),

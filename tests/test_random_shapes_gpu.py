@@ -8,23 +8,12 @@ import pytest
 import torch
 
 import eet_amd
-from eet_amd._lib import check, lib
 from eet_amd.ops import interleave_gate_up
 from oracle import ops as O
 
-from gpu_util import assert_close, gemm, mmha, stream
+from gpu_util import assert_close, gemm, gemm_fused as _fused, mmha
 
 pytestmark = pytest.mark.gpu
-
-
-def _fused(a, wp, s, M, N, K, epi, residual=None, gamma=None, eps=0.0):
-    n_out = N // 2 if epi == 2 else N
-    c = torch.empty(M, n_out, dtype=torch.float16, device=a.device)
-    check(lib().eet_gemm_w8a16_fused(a.data_ptr(), wp.data_ptr(), s.data_ptr(), c.data_ptr(), M, N, K, epi,
-                                     residual.data_ptr() if residual is not None else None,
-                                     gamma.data_ptr() if gamma is not None else None, eps, stream()),
-          "eet_gemm_w8a16_fused")
-    return c
 
 
 def _gemm_cases(n, seed):

@@ -138,6 +138,39 @@ def cpu_baseline(torch, M, hidden, d_ff, seed, budget_s=12.0):
                       f"{per_layer * 1e3:.1f} ms per layer"}
 
 
+def packer_bench(torch, eet):
+    """The offline leg, on the host: fp16 [K, N] -> int8 (per-channel /128 quantiser) -> gfx950 tile layout,
+    through the operator (`quant_weights`, threaded by column block), with the single-threaded plain-C
+    restatement of the reference quantiser timed beside it on the same matrix (it quantises only: the
+    reference's own layout pass is not restated in C).  One LLaMA-7B down-projection, K = 11008, N = 4096."""
+    import ctypes
+
+    import numpy as np
+    K, N = 11008, 4096
+    w = (torch.randn(K, N, generator=torch.Generator().manual_seed(3)) * 0.02).half()
+    eet.quant_weights(w[:64].contiguous(), torch.int8, False)     # load the library, start the threads once
+    t0 = time.perf_counter()
+    eet.quant_weights(w, torch.int8, False)
+    t_ours = time.perf_counter() - t0
+    out = {"shape": f"K={K} N={N} fp16", "quantise_and_pack_s": round(t_ours, 3),
+           "Mweights_per_s": round(K * N / t_ours / 1e6, 1), "threads": min(os.cpu_count() or 1, 16)}
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "oracle", "liboracle.so")
+    if os.path.exists(path):
+        ref = ctypes.CDLL(path)
+        ref.oracle_quantize_ref128.restype = ctypes.c_int
+        ref.oracle_quantize_ref128.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_void_p,
+                                               ctypes.c_void_p]
+        w32 = w.float().numpy()
+        q = np.empty((K, N), np.int8)
+        sc = np.empty(N, np.float32)
+        t0 = time.perf_counter()
+        ref.oracle_quantize_ref128(w32.ctypes.data, K, N, q.ctypes.data, sc.ctypes.data)
+        t_ref = time.perf_counter() - t0
+        out["cpu_port_quantise_only_s"] = round(t_ref, 3)
+        out["cpu_port_Mweights_per_s"] = round(K * N / t_ref / 1e6, 1)
+    return out
+
+
 def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed, model=LLAMA):
     """Int8 decoder of the given shape, random init: prefill `prompt` tokens then
     greedy-decode `gen` tokens; tokens/s = batch * (gen - 1) / decode time."""
@@ -392,6 +425,7 @@ def main():
         del bw
 
     if not args.no_cpu:
+        result["packer"] = packer_bench(torch, eet)
         result["cpu_baseline"] = cpu_baseline(torch, M, hidden, d_ff, seed=5)
     else:
         result["cpu_baseline"] = None

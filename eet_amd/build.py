@@ -29,7 +29,11 @@ def build(verbose=True):
     os.makedirs(os.path.join(HERE, "_obj"), exist_ok=True)
     for src in SOURCES:
         obj = os.path.join(HERE, "_obj", src + ".o")
-        cmd = [HIPCC] + [f for f in FLAGS if f != "-shared"] + ["-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+        if src.endswith(".hip"):
+            cmd = [HIPCC] + [f for f in FLAGS if f != "-shared"] + ["-x", "hip", "-c"]
+        else:   # host-only source: no device pass
+            cmd = [HIPCC, "-x", "c++", "-O3", "-std=c++17", "-fPIC", "-pthread", "-c"] + [f for f in FLAGS if f.startswith("-I")]
+        cmd += [os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

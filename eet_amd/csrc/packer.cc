@@ -58,54 +58,97 @@ void parallel_for(size_t n, size_t grain, F f)
         t.join();
 }
 
+// The three row loops below are compiled twice, for the baseline x86-64 ISA and
+// for AVX2 + F16C (chosen at load time): without F16C every fp16 -> fp32
+// conversion is a library call.  Both versions do the same IEEE operations in the
+// same order (no multiply-add pairs that could be contracted), so the results are
+// identical bit for bit.
+#define EET_ISA_CLONES __attribute__((target_clones("arch=x86-64-v3", "default")))
+
 inline float widen(float x) { return x; }
 inline float widen(_Float16 x) { return static_cast<float>(x); }
 
+template <typename T>
+inline void absmax_row(const T *row, size_t nc, float *s)
+{
+    for (size_t j = 0; j < nc; ++j) {
+        const float a = std::fabs(widen(row[j]));
+        s[j] = (s[j] < a) ? a : s[j];
+    }
+}
+
+// round-half-away-from-zero of x / s, clamped to [lo, 127]; nan_to is what a NaN
+// quotient (0 / 0 in an all-zero column) becomes.  Truncation through int32 is
+// exact once the quotient is clamped to +-200 (which cannot change the clamped
+// result), and v - trunc(v) is exact, so this equals clamp(std::round(x / s)).
+template <typename T>
+inline void quant_row(const T *row, const float *s, size_t nc, int8_t *q, float nan_to, int lo)
+{
+    for (size_t j = 0; j < nc; ++j) {
+        float v = widen(row[j]) / s[j];
+        v = (v == v) ? v : nan_to;
+        v = (v < 200.f) ? v : 200.f;
+        v = (v > -200.f) ? v : -200.f;
+        int t = static_cast<int>(v);
+        const float d = v - static_cast<float>(t);
+        t += (d >= 0.5f) ? 1 : 0;
+        t -= (d <= -0.5f) ? 1 : 0;
+        t = (t < 127) ? t : 127;
+        t = (t > lo) ? t : lo;
+        q[j] = static_cast<int8_t>(t);
+    }
+}
+
+EET_ISA_CLONES void absmax_rows_f16(const _Float16 *w, size_t K, size_t N, size_t nc, float *s)
+{
+    for (size_t k = 0; k < K; ++k)
+        absmax_row(w + k * N, nc, s);
+}
+EET_ISA_CLONES void absmax_rows_f32(const float *w, size_t K, size_t N, size_t nc, float *s)
+{
+    for (size_t k = 0; k < K; ++k)
+        absmax_row(w + k * N, nc, s);
+}
+EET_ISA_CLONES void quant_rows_f16(const _Float16 *w, size_t K, size_t N, size_t nc, const float *s, int8_t *q,
+                                   float nan_to, int lo)
+{
+    for (size_t k = 0; k < K; ++k)
+        quant_row(w + k * N, s, nc, q + k * N, nan_to, lo);
+}
+EET_ISA_CLONES void quant_rows_f32(const float *w, size_t K, size_t N, size_t nc, const float *s, int8_t *q,
+                                   float nan_to, int lo)
+{
+    for (size_t k = 0; k < K; ++k)
+        quant_row(w + k * N, s, nc, q + k * N, nan_to, lo);
+}
+inline void absmax_rows(const _Float16 *w, size_t K, size_t N, size_t nc, float *s) { absmax_rows_f16(w, K, N, nc, s); }
+inline void absmax_rows(const float *w, size_t K, size_t N, size_t nc, float *s) { absmax_rows_f32(w, K, N, nc, s); }
+inline void quant_rows(const _Float16 *w, size_t K, size_t N, size_t nc, const float *s, int8_t *q, float nan_to, int lo)
+{
+    quant_rows_f16(w, K, N, nc, s, q, nan_to, lo);
+}
+inline void quant_rows(const float *w, size_t K, size_t N, size_t nc, const float *s, int8_t *q, float nan_to, int lo)
+{
+    quant_rows_f32(w, K, N, nc, s, q, nan_to, lo);
+}
+
+// Columns [c0, c1): absmax per column, then the quotients.  EET_QUANT_REF128 is
+// the reference's quantiser (cutlass_preprocessors.cc:581-678): scale = absmax /
+// 128, clamp to [-128, 127], and an all-zero column (0 / 0) comes out as 127
+// because the reference's std::min / std::max pass NaN through to the cast that
+// way round; EET_QUANT_SYM127 divides by 127, clamps to +-127 and maps NaN to 0.
 template <typename T>
 void quantize_cols(const T *w, size_t K, size_t N, int mode, int8_t *q, T *scale, size_t c0, size_t c1)
 {
     const size_t nc = c1 - c0;
     std::vector<float> s(nc, 0.f);
-    for (size_t k = 0; k < K; ++k) {
-        const T *row = w + k * N + c0;
-        for (size_t j = 0; j < nc; ++j)
-            s[j] = std::max(s[j], std::fabs(widen(row[j])));
+    absmax_rows(w + c0, K, N, nc, s.data());
+    const bool ref = mode == EET_QUANT_REF128;
+    for (size_t j = 0; j < nc; ++j) {
+        s[j] = ref ? s[j] * (1.f / 128.f) : s[j] / 127.f;
+        scale[c0 + j] = static_cast<T>(s[j]);
     }
-    if (mode == EET_QUANT_REF128) {
-        const float r = 1.f / 128.f;
-        for (size_t j = 0; j < nc; ++j) {
-            s[j] *= r;
-            scale[c0 + j] = static_cast<T>(s[j]);
-        }
-        for (size_t k = 0; k < K; ++k) {
-            const T *row = w + k * N + c0;
-            int8_t *qr = q + k * N + c0;
-            for (size_t j = 0; j < nc; ++j) {
-                // NaN (0/0 for an all-zero column) must come out as 127: the
-                // comparisons below are false for NaN, as in std::min / std::max.
-                float v = std::round(widen(row[j]) / s[j]);
-                float c = (v < 127.f) ? v : 127.f;
-                c = (-128.f < c) ? c : -128.f;
-                qr[j] = static_cast<int8_t>(c);
-            }
-        }
-    } else {
-        for (size_t j = 0; j < nc; ++j) {
-            s[j] = s[j] / 127.f;
-            scale[c0 + j] = static_cast<T>(s[j]);
-        }
-        for (size_t k = 0; k < K; ++k) {
-            const T *row = w + k * N + c0;
-            int8_t *qr = q + k * N + c0;
-            for (size_t j = 0; j < nc; ++j) {
-                float v = std::round(widen(row[j]) / s[j]);
-                if (!(v == v))
-                    v = 0.f;
-                v = std::min(127.f, std::max(-127.f, v));
-                qr[j] = static_cast<int8_t>(v);
-            }
-        }
-    }
+    quant_rows(w + c0, K, N, nc, s.data(), q + c0, ref ? 1000.f : 0.f, ref ? -128 : -127);
 }
 
 // flat [K][N] index held by byte p of the reference's sm80 processed buffer:

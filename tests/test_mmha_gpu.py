@@ -133,3 +133,28 @@ def test_fused_rotary(gpu, dh, step):
     assert_close(ctx.cpu().numpy(), want, what="ctx")
     assert_close(kcd.cpu().numpy(), kcn, rtol=4e-3, atol=4e-3, what="k cache")   # rotated k landed in row step-1
     assert np.array_equal(vcd.cpu().numpy(), vcn)
+
+
+@pytest.mark.parametrize("B,H,step,cap,use_alibi", [(8, 32, 1152, 1153, False),      # BASELINE config 4, full size
+                                                    (32, 40, 2304, 2305, True)])     # config 5, full size
+def test_full_size_uniform_keys(gpu, B, H, step, cap, use_alibi):
+    """Size-independent property at the full benchmark shapes: when every cached key of a head equals the new
+    key, q . k_t is the same for all t, so the weights are softmax(bias) alone (uniform without ALiBi) over
+    the rows that are not padded away, and ctx is that weighted mean of V, whatever q is."""
+    dh = 128
+    g = torch.Generator(device=gpu).manual_seed(B * step)
+    k0 = torch.randn(B, H, dh, generator=g, device=gpu).half()
+    kc = k0[:, :, None, :].expand(B, H, cap, dh).contiguous()
+    vc = torch.randn(B, H, cap, dh, generator=g, device=gpu).half()
+    q = torch.randn(B, H, dh, generator=g, device=gpu).half()
+    v = torch.randn(B, H, dh, generator=g, device=gpu).half()
+    pad = torch.randint(0, step // 2, (B,), generator=g, device=gpu)
+    bias = torch.from_numpy(O.alibi_bias(H, step)).to(gpu) if use_alibi else None
+    ctx = mmha(q, k0, v, kc, vc, step, pad, bias)
+    vv = vc[:, :, :step].float()
+    vv[:, :, step - 1] = v.float()                                    # the appended row
+    logits = bias.float()[None].expand(B, H, step).clone() if use_alibi else torch.zeros(B, H, step, device=gpu)
+    logits.masked_fill_(torch.arange(step, device=gpu)[None, None, :] < pad[:, None, None], float("-inf"))
+    want = torch.einsum("bht,bhtd->bhd", torch.softmax(logits, -1), vv).reshape(B, H * dh)
+    assert_close(ctx.cpu().numpy(), want.cpu().numpy(), what="ctx")
+    assert torch.equal(kc[:, :, step - 1], k0) and torch.equal(vc[:, :, step - 1], v)

@@ -58,9 +58,9 @@ def make_weights(torch, eet, dev, layers, hidden, d_ff, seed):
         layer = {}
         for name, K, N in linear_shapes(hidden, d_ff):
             w = (torch.randn(K, N, generator=g, device=dev, dtype=torch.float32) * 0.02).half()
-            q, s = eet.quant_weights_torch(w, "ref128")
-            layer[name] = (eet.pack_weights_torch(q), s.half().contiguous())
-            del w, q
+            p, s = eet.quant_weights_device(w, False, "ref128")     # the HIP packer
+            layer[name] = (p, s)
+            del w
         out.append(layer)
     return out
 
@@ -136,6 +136,40 @@ def cpu_baseline(torch, M, hidden, d_ff, seed, budget_s=12.0):
             "sample": f"one LLaMA-7B layer (5 int8 linears, M={M}, {nbytes / 1e6:.1f} MB algorithmic), "
                       f"{reps} reps, torch {torch.__version__} dequant+matmul fp32, "
                       f"{per_layer * 1e3:.1f} ms per layer"}
+
+
+def device_packer_bench(torch, eet, lib, dev, iters=3):
+    """The packer on the GPU: eight distinct fp16 [11008, 4096] matrices (0.72 GB, more than the Infinity
+    Cache) quantised and packed round-robin.  Algorithmic bytes per matrix: read 2*K*N once, write K*N
+    packed + 2*N scales (the kernel pair reads the matrix twice: absmax first)."""
+    K, N = 11008, 4096
+    g = torch.Generator(device=dev).manual_seed(17)
+    ws = [(torch.randn(K, N, generator=g, device=dev) * 0.02).half() for _ in range(8)]
+    packed = torch.empty(K, N, dtype=torch.int8, device=dev)
+    scale = torch.empty(N, dtype=torch.float16, device=dev)
+    need = lib.eet_quantize_pack_device_workspace(N)
+    work = torch.empty(need // 4, dtype=torch.int32, device=dev)
+    st = torch.cuda.current_stream()
+
+    def call(w):
+        rc = lib.eet_quantize_pack_device(w.data_ptr(), 1, K, N, 0, None, packed.data_ptr(), scale.data_ptr(),
+                                          work.data_ptr(), need, st.cuda_stream)
+        if rc:
+            raise RuntimeError(lib.eet_last_error().decode())
+    for w in ws:
+        call(w)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(st)
+    for _ in range(iters):
+        for w in ws:
+            call(w)
+    e1.record(st)
+    torch.cuda.synchronize()
+    t = e0.elapsed_time(e1) * 1e-3 / (iters * len(ws))
+    nbytes = 3 * K * N + 2 * N
+    return {"shape": f"K={K} N={N} fp16", "us": round(t * 1e6, 1), "Gweights_per_s": round(K * N / t / 1e9, 1),
+            "GB/s": round(nbytes / t / 1e9, 1), "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4)}
 
 
 def packer_bench(torch, eet):
@@ -241,9 +275,8 @@ def prefill_gemm_bench(torch, eet, lib, dev, iters=10):
     for name, K, N in (("qkv", hidden, 3 * hidden), ("o", hidden, hidden), ("gate", hidden, d_ff),
                        ("down", d_ff, hidden)):
         w = (torch.randn(K, N, generator=g, device=dev) * 0.02).half()
-        q, s = eet.quant_weights_torch(w, "ref128")
-        p = eet.pack_weights_torch(q)
-        del w, q
+        p, s = eet.quant_weights_device(w, False, "ref128")
+        del w
         a = torch.randn(M, K, generator=g, device=dev).half()
         c = torch.empty(M, N, dtype=torch.float16, device=dev)
         args = (a.data_ptr(), p.data_ptr(), s.data_ptr(), c.data_ptr(), M, N, K, None, 0, st.cuda_stream)
@@ -411,6 +444,7 @@ def main():
     if not args.no_sweep:
         result["prefill_gemm_config3"] = prefill_gemm_bench(torch, eet, L, dev)
         result["decode_attention"] = attention_bench(torch, L, dev)
+        result["packer_device"] = device_packer_bench(torch, eet, L, dev)
 
     if args.gen > 0:
         result["decode"] = decode_bench(torch, eet, weights, dev, args.batch, args.prompt, args.gen, seed=7)

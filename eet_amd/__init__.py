@@ -4,7 +4,7 @@ the reference's own operator API."""
 from .ops import (BaichuanMmha, CrossMultiHeadAttention, Embedding, FeedForwardNetwork,  # noqa: F401
                   GatedFeedForwardNetwork, GatedFeedForwardNetworkInt8, LayerNorm, LlamaMmha,
                   MaskedMultiHeadAttention, MetaDesc, MultiHeadAttention, pack_weights,
-                  pack_weights_torch, preprocess_weights, quant_weights, quant_weights_torch,
+                  pack_weights_torch, preprocess_weights, quant_weights, quant_weights_device, quant_weights_torch,
                   unpack_weights)
 
 from .convert import (convert_baichuan_weights, convert_llama_weights, convert_name,  # noqa: F401

@@ -21,6 +21,8 @@ SIGNATURES = {
     "eet_unpack_gfx950": (_i, [_vp, _sz, _sz, _vp]),
     "eet_preprocess_ref_sm80": (_i, [_vp, _sz, _sz, _vp]),
     "eet_unprocess_ref_sm80": (_i, [_vp, _sz, _sz, _vp]),
+    "eet_quantize_pack_device_workspace": (_sz, [_sz]),
+    "eet_quantize_pack_device": (_i, [_vp, _i, _sz, _sz, _i, _vp, _vp, _vp, _vp, _sz, _vp]),
     "eet_gemm_w8a16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _vp]),
     "eet_gemm_w8a16_workspace": (_sz, [_i, _i, _i, _i]),
     "eet_gemm_w8a16_fused": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _f, _vp, _sz, _vp]),

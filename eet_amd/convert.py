@@ -63,7 +63,7 @@ def convert_name(key):
     return f"layer.{layer}.{new}" + (f".{leaf}" if leaf else "")
 
 
-def _convert(model_dict, quant_mode):
+def _convert(model_dict, quant_mode, device=None):
     out = {LAYOUT_KEY: LAYOUT_GFX950_V1}
     # fuse q, k, v of every layer in that order (modeling_llama.py:745-753)
     qkv = {}
@@ -81,10 +81,17 @@ def _convert(model_dict, quant_mode):
         work[f"layer.{layer}.self_attn.qkv_proj.weight"] = torch.cat((parts["q"], parts["k"], parts["v"]), dim=0)
     for k, v in work.items():
         if k.startswith("layer.") and k.endswith(".weight") and v.dim() == 2:
-            w = v.detach().cpu().transpose(0, 1).contiguous()          # [in, out] = [K, N]
-            if w.dtype not in (torch.float16, torch.float32):
-                w = w.float()
-            processed, scale = ops.quant_weights(w, torch.int8, False, mode=quant_mode)
+            if device is not None:   # quantise and pack on the GPU; the results stay there
+                w = v.detach().to(device).transpose(0, 1).contiguous()  # [in, out] = [K, N]
+                if w.dtype not in (torch.float16, torch.float32):
+                    w = w.float()
+                processed, scale = ops.quant_weights_device(w, False, mode=quant_mode)
+                del w
+            else:
+                w = v.detach().cpu().transpose(0, 1).contiguous()
+                if w.dtype not in (torch.float16, torch.float32):
+                    w = w.float()
+                processed, scale = ops.quant_weights(w, torch.int8, False, mode=quant_mode)
             out[k] = processed
             out[k[: -len(".weight")] + ".scale"] = scale
         else:
@@ -92,18 +99,20 @@ def _convert(model_dict, quant_mode):
     return out
 
 
-def convert_llama_weights(model_dict, data_type=torch.int8, model_attr="model", quant_mode="ref128"):
-    """HF LLaMA state dict -> operator state dict (int8 weight-only)."""
+def convert_llama_weights(model_dict, data_type=torch.int8, model_attr="model", quant_mode="ref128", device=None):
+    """HF LLaMA state dict -> operator state dict (int8 weight-only).  With
+    device="cuda:0" the linears are quantised and packed by the HIP packer and
+    returned as GPU tensors (same bits as the host path)."""
     if data_type != torch.int8:
         raise NotImplementedError("[EET][ERROR] only the int8 weight-only conversion is implemented")
-    return _convert(dict(model_dict), quant_mode)
+    return _convert(dict(model_dict), quant_mode, device)
 
 
-def convert_baichuan_weights(model_dict, data_type=torch.int8, model_attr="model", quant_mode="ref128"):
-    """HF Baichuan state dict (fused W_pack) -> operator state dict (int8 weight-only)."""
+def convert_baichuan_weights(model_dict, data_type=torch.int8, model_attr="model", quant_mode="ref128", device=None):
+    """HF Baichuan state dict (fused W_pack) -> operator state dict (int8 weight-only); device as above."""
     if data_type != torch.int8:
         raise NotImplementedError("[EET][ERROR] only the int8 weight-only conversion is implemented")
-    return _convert(dict(model_dict), quant_mode)
+    return _convert(dict(model_dict), quant_mode, device)
 
 
 def repack_reference_state_dict(ref_dict):

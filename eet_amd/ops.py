@@ -491,6 +491,30 @@ def quant_weights_torch(w, mode="ref128"):
     return r.to(torch.int8), s32.to(w.dtype)
 
 
+def quant_weights_device(origin_weight, return_unprocessed_quantized_tensor=False, mode="ref128"):
+    """quant_weights for a weight that already lives on the GPU (fp16 / fp32
+    [K, N], K % 64 == 0, N % 16 == 0): two HIP kernels instead of the host
+    threads, same bits.  Returns [processed, scales] or [unprocessed,
+    processed, scales] like quant_weights, as GPU tensors.  The reference
+    only quantises CPU tensors (fpA_intB_gemm_wrapper.cu:33)."""
+    w = origin_weight
+    if w.device.type != "cuda" or w.dim() != 2 or not w.is_contiguous() or w.dtype not in (torch.float16, torch.float32):
+        raise RuntimeError("[EET][ERROR] quant_weights_device: expected a contiguous fp16 / fp32 GPU tensor [K, N]")
+    K, N = w.shape
+    L = lib()
+    packed = torch.empty(K, N, dtype=torch.int8, device=w.device)
+    scales = torch.empty(N, dtype=w.dtype, device=w.device)
+    q = torch.empty(K, N, dtype=torch.int8, device=w.device) if return_unprocessed_quantized_tensor else None
+    need = L.eet_quantize_pack_device_workspace(N)
+    ws = workspaces.get("quant_absmax", max(need // 4, 1), torch.int32, w.device)
+    with torch.cuda.device(w.device):
+        check(L.eet_quantize_pack_device(w.data_ptr(), 0 if w.dtype == torch.float32 else 1, K, N,
+                                         {"ref128": 0, "sym127": 1}[mode], q.data_ptr() if q is not None else None,
+                                         packed.data_ptr(), scales.data_ptr(), ws.data_ptr(), need, _stream()),
+              "eet_quantize_pack_device")
+    return [q, packed, scales] if return_unprocessed_quantized_tensor else [packed, scales]
+
+
 def quant_weights(origin_weight, quant_type, return_unprocessed_quantized_tensor=False, mode="ref128"):
     """symmetric_quantize_last_axis_of_tensor
     (3rdparty/cutlass_kernels/fpA_intB_gemm_wrapper.cu:26-105).  Returns

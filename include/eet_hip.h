@@ -81,6 +81,20 @@ int eet_unprocess_ref_sm80(const int8_t *processed, size_t K, size_t N, int8_t *
  * Device kernels (gfx950).
  * ---------------------------------------------------------------------- */
 
+/* The packer on the GPU, for weights that already live in HBM: w[K][N]
+ * (row-major, w_dtype as above, K % 64 == 0, N % 16 == 0) -> packed[K][N] in the
+ * gfx950 layout, scale[N] in w's dtype and, when q is not NULL, the
+ * unprocessed q[K][N]; all device pointers.  Bit-identical to
+ * eet_quantize_int8 followed by eet_pack_gfx950 in both modes.  workspace:
+ * eet_quantize_pack_device_workspace(N) bytes of device memory.  The reference
+ * quantises on one host core only (cutlass_preprocessors.cc:581-678, reached
+ * from fpA_intB_gemm_wrapper.cu:26-105, which rejects CUDA tensors at :33);
+ * this entry point has no counterpart there. */
+size_t eet_quantize_pack_device_workspace(size_t N);
+int eet_quantize_pack_device(const void *w, int w_dtype, size_t K, size_t N, int mode,
+                             int8_t *q, int8_t *packed, void *scale, void *workspace,
+                             size_t workspace_bytes, void *stream);
+
 /* C[M][N] (half) = A[M][K] (half) . (int8 W[K][N] * scale[N] (half)), fp32
  * accumulation, one rounding to half.  Wpacked comes from eet_pack_gfx950.
  * M <= 32 takes the HBM-streaming small-M kernel, larger M the LDS-staged MFMA

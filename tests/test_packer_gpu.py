@@ -104,3 +104,29 @@ def test_arguments(gpu):
     torch.cuda.synchronize()
     with pytest.raises(RuntimeError):
         eet_amd.quant_weights_device(torch.zeros(64, 16))  # CPU tensor
+
+
+def test_converter_on_device(gpu):
+    """convert_llama_weights(device=...) quantises and packs with the HIP packer: same keys and bits as the
+    host conversion, linears left on the GPU."""
+    from eet_amd import convert
+    hid, ff = 128, 192
+    g = torch.Generator().manual_seed(3)
+    r = lambda *s: (torch.randn(*s, generator=g) * 0.05).half()
+    sd = {"model.embed_tokens.weight": r(50, hid), "model.norm.weight": r(hid), "lm_head.weight": r(50, hid)}
+    p = "model.layers.0."
+    for n in "qkvo":
+        sd[p + f"self_attn.{n}_proj.weight"] = r(hid, hid)
+    sd[p + "mlp.gate_proj.weight"], sd[p + "mlp.up_proj.weight"] = r(ff, hid), r(ff, hid)
+    sd[p + "mlp.down_proj.weight"] = r(hid, ff)
+    sd[p + "input_layernorm.weight"], sd[p + "post_attention_layernorm.weight"] = r(hid), r(hid)
+    host = convert.convert_llama_weights(sd)
+    dev = convert.convert_llama_weights(sd, device=gpu)
+    assert host.keys() == dev.keys()
+    for k, v in host.items():
+        if isinstance(v, torch.Tensor):
+            assert torch.equal(dev[k].cpu(), v), k
+            if k.endswith("proj.weight") or k.startswith("layer.0.ffn.") and k.endswith(("weight", "scale")) and "layernorm" not in k:
+                assert dev[k].device.type == "cuda", k
+        else:
+            assert dev[k] == v

@@ -131,19 +131,21 @@ __device__ __forceinline__ int quant_fast(float x, float s, float inv_s, float n
 }
 
 // One k-tile (64 rows) x 128 columns per workgroup: rows are read in 256-byte
-// (fp16) pieces, quantised into an LDS tile, and leave as eight whole 1 KiB
-// packed tiles: byte 16*(16*g + i) + b of tile (nt, kt) is
-// q[64*kt + 16*g + b][16*nt + i] ^ 0x80 (the layout of eet_pack_gfx950).
+// (fp16) pieces and quantised; the tile is kept column-major in LDS (a thread
+// owns 4 consecutive rows of its 8 columns, i.e. 8 whole 32-bit words), so that
+// the 16 bytes lane (g, i) of a packed tile holds -- q[64*kt + 16*g + b][16*nt
+// + i] ^ 0x80 for b = 0 .. 15, the layout of eet_pack_gfx950 -- are four
+// consecutive words, and the tile leaves as eight whole 1 KiB packed tiles.
 template <typename T>
 __global__ __launch_bounds__(256) void quant_pack_kernel(const T *__restrict__ w, size_t K, size_t N, int ref128,
                                                          const uint32_t *__restrict__ amax, int8_t *__restrict__ q_out,
                                                          uint8_t *__restrict__ packed, T *__restrict__ scale)
 {
-    __shared__ __attribute__((aligned(16))) int8_t lq[64][kTileCols + 16];   // +16: rows land in different banks
+    __shared__ uint32_t lq[kTileCols][17];   // [column][4-row word], one word of padding per column
     const size_t kt = blockIdx.y, ktiles = K / 64;
     const size_t col0 = (size_t)blockIdx.x * kTileCols;
     const int tid = threadIdx.x;
-    const int c8 = (tid & 15) * 8;
+    const int c8 = (tid & 15) * 8, rw = tid >> 4;   // columns c8 .. c8+7, rows 4*rw .. 4*rw+3
     const size_t col = col0 + c8;
     const float nan_to = ref128 ? 1000.f : 0.f;
     const int lo = ref128 ? -128 : -127;
@@ -163,22 +165,29 @@ __global__ __launch_bounds__(256) void quant_pack_kernel(const T *__restrict__ w
             for (int i = 0; i < 8; ++i)
                 scale[col + i] = static_cast<T>(s[i]);
         }
+        T v[4][8];
+#pragma unroll
+        for (int it = 0; it < 4; ++it)
+            __builtin_memcpy(v[it], w + (kt * 64 + 4 * rw + it) * N + col, sizeof(v[it]));
+        uint32_t word[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
-            const int row = it * 16 + (tid >> 4);
-            T v[8];
-            __builtin_memcpy(v, w + (kt * 64 + row) * N + col, sizeof(v));
             union {
                 int8_t b[8];
                 u32x2 u;
             } o;
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                o.b[i] = static_cast<int8_t>(quant_fast(to_f32(v[i]), s[i], inv_s[i], nan_to, lo));
-            *reinterpret_cast<u32x2 *>(&lq[row][c8]) = o.u;
+            for (int i = 0; i < 8; ++i) {
+                const int t = quant_fast(to_f32(v[it][i]), s[i], inv_s[i], nan_to, lo);
+                o.b[i] = static_cast<int8_t>(t);
+                word[i] |= (static_cast<uint32_t>(t) & 0xffu) << (8 * it);
+            }
             if (q_out != nullptr)
-                *reinterpret_cast<u32x2 *>(q_out + (kt * 64 + row) * N + col) = o.u;
+                *reinterpret_cast<u32x2 *>(q_out + (kt * 64 + 4 * rw + it) * N + col) = o.u;
         }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            lq[c8 + i][rw] = word[i] ^ 0x80808080u;
     }
     __syncthreads();
     // 8 tiles x 64 lanes = 512 pieces of 16 bytes, two per thread
@@ -190,14 +199,9 @@ __global__ __launch_bounds__(256) void quant_pack_kernel(const T *__restrict__ w
         const size_t nt = col0 / 16 + n8;
         if (nt * 16 >= N)
             continue;
-        union {
-            uint8_t b[16];
-            u32x4 u;
-        } o;
-#pragma unroll
-        for (int b = 0; b < 16; ++b)
-            o.b[b] = static_cast<uint8_t>(lq[g * 16 + b][n8 * 16 + i]) ^ 0x80u;
-        *reinterpret_cast<u32x4 *>(packed + (nt * ktiles + kt) * 1024 + lane * 16) = o.u;
+        const uint32_t *src = &lq[n8 * 16 + i][4 * g];
+        const u32x4 o = {src[0], src[1], src[2], src[3]};
+        *reinterpret_cast<u32x4 *>(packed + (nt * ktiles + kt) * 1024 + lane * 16) = o;
     }
 }
 

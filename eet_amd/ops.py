@@ -28,8 +28,17 @@ def _ptr(t):
     return t.data_ptr() if t is not None and t.numel() > 0 else None
 
 
+def _current_stream():
+    """Handle of torch's current stream on the current device (the private
+    accessor when torch has it: it costs a tenth of building a Stream object)."""
+    try:
+        return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
+    except AttributeError:
+        return torch.cuda.current_stream().cuda_stream
+
+
 def _stream():
-    return _StreamScope.handle if _StreamScope.handle is not None else torch.cuda.current_stream().cuda_stream
+    return _StreamScope.handle if _StreamScope.handle is not None else _current_stream()
 
 
 class _StreamScope:
@@ -37,7 +46,7 @@ class _StreamScope:
     handle = None
 
     def __enter__(self):
-        _StreamScope.handle = torch.cuda.current_stream().cuda_stream
+        _StreamScope.handle = _current_stream()
 
     def __exit__(self, *a):
         _StreamScope.handle = None
@@ -276,6 +285,26 @@ class _MmhaInt8:
         qbuf = workspaces.get("q_buf", desc.batch_size * max(desc.max_seq_len, 1) * self.inner, f16, dev)
         cbuf = workspaces.get("context_buf", desc.batch_size * max(desc.max_seq_len, 1) * self.inner, f16, dev)
         out = workspaces.get("self_mask_attn_cache", desc.batch_size * max(desc.max_seq_len, 1) * hidden, f16, dev)
+        if not first_pass and M <= RMS_FUSE_MAX_M:
+            # the whole incremental call from one library call: RMSnorm + QKV, rotary + append +
+            # attention, output projection + residual
+            alibi = None
+            if bias is not None:
+                if bias.numel() != H * self.step:
+                    raise RuntimeError(f"[EET][ERROR] {self._name}: relative_attention_bias must be [H, 1, step] "
+                                       f"with step={self.step}, got {tuple(bias.shape)}")
+                alibi = bias.to(f16).contiguous()
+            need = L.eet_mmha_int8_decode_workspace(B, H, dh, self.step)
+            ws = workspaces.get("mmha_ws", max(need // 4, 1), torch.float32, dev)
+            rope = self.rope_table.data_ptr() + (self.step - 1) * dh * 4 if self._rope else None
+            check(L.eet_mmha_int8_decode(x.data_ptr(), self.gamma.data_ptr(), desc.layernorm_eps,
+                                         self.qkv_w.data_ptr(), self.qkv_s.data_ptr(), self.o_w.data_ptr(),
+                                         self.o_s.data_ptr(), self.k_cache.data_ptr(), self.v_cache.data_ptr(),
+                                         _ptr(alibi), _ptr(pad), rope, qkv.data_ptr(), cbuf.data_ptr(),
+                                         out.data_ptr(), B, H, dh, hidden, self.step, self.t_cap, ws.data_ptr(),
+                                         ws.numel() * 4, _stream()), "eet_mmha_int8_decode")
+            self._keep = (x, pad, alibi, reorder)  # inputs of kernels still in flight
+            return out[: M * hidden].view(B, S, hidden)
         if M <= RMS_FUSE_MAX_M:
             # RMSnorm folded into the GEMM's activation load
             _gemm(x, self.qkv_w, self.qkv_s, qkv, M, 3 * self.inner, hidden, EPI_NONE, None, self.gamma,
@@ -391,13 +420,17 @@ class GatedFeedForwardNetworkInt8:
         act = workspaces.get("ffn_inner_act", cap * self.d_ff, f16, dev)
         out = workspaces.get(self.cache_name, cap * hidden, f16, dev)
         # fc1, fc2 and gated_act (gated_ffn_int8.cpp:253-301, 168-179) in one launch; at decode
-        # sizes the RMSnorm (:112) rides in the same launch
+        # sizes the RMSnorm (:112) rides in the same launch and fc3 follows from the same library call
         if M <= RMS_FUSE_MAX_M:
-            _gemm(x, self.w01, self.s01, act, M, 2 * self.d_ff, hidden, EPI_SWIGLU, None, self.gamma,
-                  desc.layernorm_eps)
-        else:
-            _rmsnorm(x, self.gamma, xn, M, hidden, desc.layernorm_eps)
-            _gemm(xn, self.w01, self.s01, act, M, 2 * self.d_ff, hidden, EPI_SWIGLU)
+            check(lib().eet_gated_ffn_int8_decode(x.data_ptr(), self.gamma.data_ptr(), desc.layernorm_eps,
+                                                  self.w01.data_ptr(), self.s01.data_ptr(), self.w2.data_ptr(),
+                                                  self.s2.data_ptr(), act.data_ptr(), out.data_ptr(), M, hidden,
+                                                  self.d_ff, 1 if add_residual else 0, _stream()),
+                  "eet_gated_ffn_int8_decode")
+            self._keep = x
+            return out[: M * hidden].view(B, S, hidden)
+        _rmsnorm(x, self.gamma, xn, M, hidden, desc.layernorm_eps)
+        _gemm(xn, self.w01, self.s01, act, M, 2 * self.d_ff, hidden, EPI_SWIGLU)
         # fc3 with add_input_bias_layernorm's residual add (:303-357) in its epilogue
         if add_residual:
             _gemm(act, self.w2, self.s2, out, M, hidden, self.d_ff, EPI_RESIDUAL, x)

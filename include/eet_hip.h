@@ -201,6 +201,35 @@ int eet_kv_cache_reorder(const void *k_src, const void *v_src, void *k_dst, void
                          const int64_t *reorder_index, int B, int H, int dh, int rows, int T_cap,
                          void *stream);
 
+/* One incremental call (one new token per sequence, B <= 32) of the attention
+ * sub-layer, all launches from one call: RMSnorm + QKV projection, rotary (when
+ * rope_cos_sin is given) + cache append + masked attention, output projection +
+ * residual.  x [B][hidden] is both the input and the residual; qkv_buf
+ * [B][3*H*dh] and ctx_buf [B][H*dh] are scratch; out [B][hidden] must not
+ * alias x.  Weights are packed int8 [hidden][3*H*dh] and [H*dh][hidden] with
+ * their fp16 scales; the other arguments are those of eet_mmha_decode.
+ * Replaces LlamaMmha::forward_inc (csrc/op/llama_mmha.cpp:202-266) and
+ * BaichuanMmha::forward_inc (csrc/op/baichuan_mmha.cpp:166-216) without the
+ * beam reorder, which stays a separate call (eet_kv_cache_reorder). */
+size_t eet_mmha_int8_decode_workspace(int B, int H, int dh, int step);
+int eet_mmha_int8_decode(const void *x, const void *rms_gamma, float rms_eps, const void *qkv_w,
+                         const void *qkv_scale, const void *o_w, const void *o_scale,
+                         void *k_cache, void *v_cache, const void *alibi, const int64_t *pad,
+                         const float *rope_cos_sin, void *qkv_buf, void *ctx_buf, void *out,
+                         int B, int H, int dh, int hidden, int step, int T_cap, void *workspace,
+                         size_t workspace_bytes, void *stream);
+
+/* The gated FFN sub-layer for B <= 32 rows, both launches from one call:
+ * RMSnorm + gate and up projections + SwiGLU (w01 / scale01: gate and up
+ * interleaved by 16-channel tile, [hidden][2*d_ff]), then the down projection
+ * (+ x when add_residual).  act_buf [B][d_ff] is scratch; out [B][hidden] must
+ * not alias x.  Replaces GatedFeedForwardNetworkInt8::forward
+ * (csrc/op/gated_ffn_int8.cpp:98-132) at decode sizes. */
+int eet_gated_ffn_int8_decode(const void *x, const void *rms_gamma, float rms_eps, const void *w01,
+                              const void *scale01, const void *w2, const void *scale2,
+                              void *act_buf, void *out, int B, int hidden, int d_ff,
+                              int add_residual, void *stream);
+
 /* Causal prefill attention over the prompt, reading K and V from the caches
  * filled by eet_qkv_split.  q [B][H][S][dh]; ctx [B][S][H*dh]; alibi NULL or
  * [H][S] half (slope * j, the diagonal row of the reference's mask); pad as in

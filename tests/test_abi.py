@@ -73,6 +73,16 @@ def test_device_entry_points_validate_before_launch():
     need = L.eet_mmha_decode_workspace(1, 8, 128, 1100)           # fewer heads than CUs: the time axis is split
     assert need > 0
     assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 8, 128, 1100, 1153, None, None, 0, None) == -4
+    # operator-level decode calls: argument checks happen before any launch
+    assert L.eet_mmha_int8_decode(None, p, 1e-6, p, p, p, p, p, p, None, None, None, p, p, p, 1, 1, 128, 128, 1, 8,
+                                  None, 0, None) == -1
+    assert L.eet_mmha_int8_decode(p, p, 1e-6, p, p, p, p, p, p, None, None, None, p, p, p, 33, 1, 128, 128, 1, 8,
+                                  None, 0, None) == -2                       # more than 32 rows
+    assert L.eet_mmha_int8_decode(p, p, 1e-6, p, p, p, p, p, p, None, None, None, p, p, p, 1, 1, 128, 128, 1, 8,
+                                  None, 0, None) == -1                       # out aliases x
+    assert L.eet_gated_ffn_int8_decode(p, p, 1e-6, p, p, p, p, p, None, 1, 128, 256, 1, None) == -1
+    assert L.eet_gated_ffn_int8_decode(p, p, 1e-6, p, p, p, p, p, p, 40, 128, 256, 1, None) == -2
+    assert L.eet_mmha_int8_decode_workspace(8, 32, 128, 1100) == L.eet_mmha_decode_workspace(8, 32, 128, 1100)
     assert L.eet_rope_table(None, 4, 128, None) == -1
     assert L.eet_rmsnorm(p, p, p, 1, 20000, 1e-6, None) == -2
     assert L.eet_qkv_split(p, p, p, p, 1, 4, 1, 128, 1, -1, 6, 8, None) == -1  # rows past the cache end

@@ -51,21 +51,22 @@ __device__ __forceinline__ float group_sum(float v)
 }
 
 // NeoX rotary on one 8-element slice.  x holds elements d = 8*sub .. 8*sub+7 of
-// a head row, y the slice DH/2 away; rope_row is [cos(DH/2) | sin(DH/2)] for the
-// position.  fp32 math, one rounding to fp16 (csrc/core/common.cuh:209-225).
+// a head row, y the slice DH/2 away; cs / sn are cos and sin of the position for
+// the slice's 8 pairs (entries (sub % (DH/16)) * 8 .. of the table row
+// [cos(DH/2) | sin(DH/2)]).  fp32 math, one rounding to fp16
+// (csrc/core/common.cuh:209-225).
 template <int DH>
-__device__ __forceinline__ u32x4 rotate8(const u32x4 &x, const u32x4 &y, int sub, const float *rope_row)
+__device__ __forceinline__ u32x4 rotate8(const u32x4 &x, const u32x4 &y, int sub, const float (&cs)[8],
+                                         const float (&sn)[8])
 {
     constexpr int LPR = DH / 8;
     const bool lower = sub < LPR / 2;
-    const int i0 = (sub % (LPR / 2)) * 8;
     const half8 hx = __builtin_bit_cast(half8, x), hy = __builtin_bit_cast(half8, y);
     half8 o;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        const float c = rope_row[i0 + e], sn = rope_row[DH / 2 + i0 + e];
         const float a = (float)hx[e], b = (float)hy[e];
-        o[e] = (_Float16)(lower ? a * c - b * sn : a * c + b * sn);
+        o[e] = (_Float16)(lower ? a * cs[e] - b * sn[e] : a * cs[e] + b * sn[e]);
     }
     return __builtin_bit_cast(u32x4, o);
 }
@@ -113,30 +114,43 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
     // appends it all the same, as the reference does, and gives it no weight.)
     const bool own_last = k_new != nullptr && step - 1 >= t0 && step - 1 < t1;
     const bool append = own_last || (k_new != nullptr && span == 0 && split == 0);
-    u32x4 knew = {0, 0, 0, 0}, vnew = {0, 0, 0, 0};
-    if (append) {
-        knew = *reinterpret_cast<const u32x4 *>(k_new + qoff + sub * 8);
-        if (rope_row != nullptr) {
-            const u32x4 ky = *reinterpret_cast<const u32x4 *>(k_new + qoff + (sub ^ (LPR / 2)) * 8);
-            knew = rotate8<DH>(knew, ky, sub, rope_row);
-        }
-        vnew = *reinterpret_cast<const u32x4 *>(v_new + qoff + sub * 8);
-        if (rs == 0) {
-            *reinterpret_cast<u32x4 *>(kc + (size_t)(step - 1) * DH + sub * 8) = knew;
-            *reinterpret_cast<u32x4 *>(vc + (size_t)(step - 1) * DH + sub * 8) = vnew;
-        }
-    }
+    // The requests for the new token's q, k, v and the rotary row go out first and
+    // are consumed only after the first cache rows have been requested as well
+    // (below), so the two memory latencies overlap.
+    // They go through buffer resources of size zero when there is nothing to read
+    // (no append, no rotary row): zeros come back and no branch surrounds the loads.
     const int r_last = own_last ? step - 1 - t0 : -1;
-
-    u32x4 qv = *reinterpret_cast<const u32x4 *>(q + qoff + sub * 8);
-    if (rope_row != nullptr) {
-        u32x4 qy;
-        qy.x = __shfl_xor(qv.x, LPR / 2, 64);
-        qy.y = __shfl_xor(qv.y, LPR / 2, 64);
-        qy.z = __shfl_xor(qv.z, LPR / 2, 64);
-        qy.w = __shfl_xor(qv.w, LPR / 2, 64);
-        qv = rotate8<DH>(qv, qy, sub, rope_row);
+    u32x4 knew, kpair, vnew, qv;
+    float rcs[8], rsn[8];
+#if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
+    {
+        const unsigned row_bytes = append ? (unsigned)(DH * 2) : 0u;
+        const __amdgpu_buffer_rsrc_t knr = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<_Float16 *>(append ? k_new + qoff : q), 0, row_bytes, 0x00020000);
+        const __amdgpu_buffer_rsrc_t vnr = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<_Float16 *>(append ? v_new + qoff : q), 0, row_bytes, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rpr = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float *>(rope_row ? rope_row : reinterpret_cast<const float *>(q)), 0,
+            rope_row ? (unsigned)(DH * 4) : 0u, 0x00020000);
+        const int i0 = (sub % (LPR / 2)) * 8;
+        knew = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(knr, sub * 16, 0, 0));
+        kpair = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(knr, (sub ^ (LPR / 2)) * 16, 0, 0));
+        vnew = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(vnr, sub * 16, 0, 0));
+        qv = *reinterpret_cast<const u32x4 *>(q + qoff + sub * 8);
+        const u32x4 c0 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, i0 * 4, 0, 0));
+        const u32x4 c1 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, i0 * 4 + 16, 0, 0));
+        const u32x4 s0 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, (DH / 2 + i0) * 4, 0, 0));
+        const u32x4 s1 =
+            __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, (DH / 2 + i0) * 4 + 16, 0, 0));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            rcs[e] = __uint_as_float(c0[e]);
+            rcs[4 + e] = __uint_as_float(c1[e]);
+            rsn[e] = __uint_as_float(s0[e]);
+            rsn[4 + e] = __uint_as_float(s1[e]);
+        }
     }
+#endif
 
     // Every group of LPR lanes walks its own stream of rows (rs, rs + RPB, ...)
     // with a running softmax (max m, sum l, un-normalised acc).  The K and V rows
@@ -158,38 +172,60 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
         0x00020000);
     constexpr int kStream = 2;  // aux bits of a buffer load: non-temporal (every row is read exactly once)
     auto row_off = [&](int i) { return (unsigned)((rs + i * RPB) * (DH * 2) + sub * 16); };
-    // The first pass of the loop (i0 = -UN) only fills the ring: there is no separate
-    // prologue, so the wait before each slot is the same on every pass (all but the
-    // UN-1 newer slots' requests) instead of the merge with a differently ordered
-    // prologue, which drained the ring once per pass.
+    // Slot u is consumed first and refilled afterwards, so a slot's registers are
+    // never live twice and the compiler keeps every slot in place: with the refill
+    // ahead of the use it moved freshly requested registers at the end of each pass,
+    // which waits for them and empties the ring.  The bias term sits in a 32-bit
+    // register per slot (sign-extending load): pairs of 16-bit values get packed,
+    // which is a move of a pending load again.
     u32x4 kv[UN], vv[UN];
-    unsigned short ab[UN];
+    int ab[UN];
+    auto request = [&](int u, int i) {
+        kv[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(krs, row_off(i), 0, kStream));
+        vv[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(vrs, row_off(i), 0, kStream));
+        ab[u] = (int)(short)__builtin_amdgcn_raw_buffer_load_b16(ars, (unsigned)((rs + i * RPB) * 2), 0, 0);
+    };
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-        kv[u] = u32x4{0, 0, 0, 0};
-        vv[u] = u32x4{0, 0, 0, 0};
-        ab[u] = 0;
+        request(u, u);
+        __builtin_amdgcn_sched_barrier(0);
     }
+    // Now the new token: rotate and append k, rotate q.  Their requests are older
+    // than the ring's, so waiting for them leaves the ring in flight.
+    {
+        const u32x4 krot = rotate8<DH>(knew, kpair, sub, rcs, rsn);
+        u32x4 qy;
+        qy.x = __shfl_xor(qv.x, LPR / 2, 64);
+        qy.y = __shfl_xor(qv.y, LPR / 2, 64);
+        qy.z = __shfl_xor(qv.z, LPR / 2, 64);
+        qy.w = __shfl_xor(qv.w, LPR / 2, 64);
+        const u32x4 qrot = rotate8<DH>(qv, qy, sub, rcs, rsn);
+        if (rope_row != nullptr) {
+            knew = krot;
+            qv = qrot;
+        }
+        if (append && rs == 0) {
+            *reinterpret_cast<u32x4 *>(kc + (size_t)(step - 1) * DH + sub * 8) = knew;
+            *reinterpret_cast<u32x4 *>(vc + (size_t)(step - 1) * DH + sub * 8) = vnew;
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
     float m_run = -INFINITY, l_run = 0.f;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const int iters = (n + RPB - 1) / RPB;  // the same for every stream of the workgroup
-    for (int i0 = -UN; i0 < iters; i0 += UN) {
+    for (int i0 = 0; i0 < iters; i0 += UN) {
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             const int r = rs + (i0 + u) * RPB;  // the same for all LPR lanes of a group
-            u32x4 kcur = kv[u], vcur = vv[u];
-            const unsigned short acur = ab[u];
-            kv[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(krs, row_off(i0 + u + UN), 0, kStream));
-            vv[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(vrs, row_off(i0 + u + UN), 0, kStream));
-            ab[u] = __builtin_amdgcn_raw_buffer_load_b16(ars, (unsigned)((rs + (i0 + u + UN) * RPB) * 2), 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            if (r == r_last) {  // the row being appended by this launch is still in registers
-                kcur = knew;
-                vcur = vnew;
-            }
-            float d = group_sum<LPR>(dot8(qv, kcur)) * scale;
-            if (r >= 0 && r < n) {
-                d += (float)__builtin_bit_cast(_Float16, acur);  // 0 without ALiBi
+            if (r < n) {   // uniform over the LPR lanes of a group, so the group sum below is whole
+                u32x4 kcur = kv[u], vcur = vv[u];
+                if (r == r_last) {  // the row being appended by this launch is still in registers
+                    kcur = knew;
+                    vcur = vnew;
+                }
+                float d = group_sum<LPR>(dot8(qv, kcur)) * scale;
+                d += (float)__builtin_bit_cast(_Float16, (unsigned short)ab[u]);  // 0 without ALiBi
                 const float m_new = fmaxf(m_run, d);
                 const float c = __expf(m_run - m_new);  // 0 on the first row (m_run = -inf)
                 const float p = __expf(d - m_new);
@@ -200,6 +236,9 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
                     acc[e] = acc[e] * c + p * (float)hv[e];
                 m_run = m_new;
             }
+            __builtin_amdgcn_sched_barrier(0);
+            request(u, i0 + u + UN);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 #else

@@ -48,30 +48,44 @@ struct Batch {
 // operand straight from the row-major matrix instead costs 16 half-used lines
 // per instruction and measured 1.4 us (M = 8) to 2.5 us (M = 16) on a 4 us
 // kernel.
+//
+// The weights come through a buffer resource over the whole packed matrix: the
+// n-tile and k-tile select a wavefront-uniform (scalar) offset, the lane adds
+// 16 * lane.  With `valid` false (the request one batch past the end, which the
+// main loop issues without a branch so that its waits stay exact) the lane
+// offset is moved out of range: zeros come back and no memory is touched; the
+// activations then re-read k-tile 0.
+#if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
 template <int NT, int RG, int WAVES, int U, bool RMS>
-__device__ __forceinline__ void load_batch(Batch<NT, RG, U> &b, const u32x4 *const (&wbase)[NT],
-                                           const u32x4 *const (&abase)[RG], const u32x4 *gbase, int kt)
+__device__ __forceinline__ void load_batch(Batch<NT, RG, U> &b, __amdgpu_buffer_rsrc_t wrsrc,
+                                           const unsigned (&wtile)[NT], int lane, const u32x4 *const (&abase)[RG],
+                                           const u32x4 *gbase, int kt, bool valid)
 {
+    constexpr int kStream = 2;  // aux bits: non-temporal (every weight is read exactly once)
+    const unsigned voff = valid ? (unsigned)lane * 16u : 0x80000000u;
     // All weight loads (HBM latency) go out first, then the activation loads
     // (L2 hits); loads return in issue order.
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-            b.w[u][t] = __builtin_nontemporal_load(wbase[t] + (size_t)(kt + u * WAVES) * 64);
+            b.w[u][t] = __builtin_bit_cast(
+                u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, voff, wtile[t] + (unsigned)(kt + u * WAVES) * 1024u,
+                                                             kStream));
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int r = 0; r < RG; ++r)
-            b.a[u][r] = abase[r][(kt + u * WAVES) * 8];
+            b.a[u][r] = abase[r][valid ? (kt + u * WAVES) * 8 : 0];
     if (RMS) {
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            b.gam[u] = gbase[(kt + u * WAVES) * 8];
+            b.gam[u] = gbase[valid ? (kt + u * WAVES) * 8 : 0];
     }
     __builtin_amdgcn_sched_barrier(0);
 }
+#endif
 
 // The row-wise activation pieces are turned into MFMA operands through a
 // wavefront-private LDS slab: lane (g, j) of operand half h needs piece
@@ -139,9 +153,10 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     _Float16 *__restrict__ C, int M, int N, int K, const _Float16 *__restrict__ residual, int epi,
     const _Float16 *__restrict__ rms_gamma, float rms_eps)
 {
+#if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
     constexpr int MT = (RG + 1) / 2;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: feeds scalar offsets
     const int g = lane >> 4, j = lane & 15;
     const int ktiles = K >> 6;
     const int ntiles = N >> 4;
@@ -167,12 +182,12 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
             acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     // A tile index past the end is clamped: its results are never written.
-    const u32x4 *wbase[NT];
+    const __amdgpu_buffer_rsrc_t wrsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4 *>(Wp), 0, (unsigned)((size_t)K * N), 0x00020000);
+    unsigned wtile[NT];  // byte offset of the n-tile's first k-tile
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        int nt = min(nt0 + t, ntiles - 1);
-        wbase[t] = Wp + (size_t)nt * ktiles * 64 + lane;
-    }
+    for (int t = 0; t < NT; ++t)
+        wtile[t] = (unsigned)min(nt0 + t, ntiles - 1) * (unsigned)ktiles * 1024u;
     // Rows past M read row M-1: column m of the product depends only on
     // activation row m, and rows >= M are not written.
     const u32x4 *abase[RG];
@@ -217,21 +232,22 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
 
     // This wavefront's k-tiles are wave, wave + WAVES, ...; they are taken in
     // batches of U with the next batch's loads in flight while the current one
-    // is multiplied (two register buffers).
+    // is multiplied (two register buffers).  The request for the batch after
+    // next is issued on every pass, past the end too (where it costs nothing):
+    // with a branch around it the compiler has to wait for that request as well
+    // before the second multiply, i.e. it empties the pipeline once per pass.
     const int mine = (ktiles - wave + WAVES - 1) / WAVES;
     const int nbatch = mine / U;
     constexpr int STEP = U * WAVES;
     int kt = wave;
     {
         Batch<NT, RG, U> b0, b1;
-        if (nbatch > 0)
-            load_batch<NT, RG, WAVES, U, RMS>(b0, wbase, abase, gbase, kt);
+        load_batch<NT, RG, WAVES, U, RMS>(b0, wrsrc, wtile, lane, abase, gbase, kt, nbatch > 0);
         int i = 0;
         for (; i + 2 <= nbatch; i += 2) {
-            load_batch<NT, RG, WAVES, U, RMS>(b1, wbase, abase, gbase, kt + STEP);
+            load_batch<NT, RG, WAVES, U, RMS>(b1, wrsrc, wtile, lane, abase, gbase, kt + STEP, true);
             mma_batch<NT, RG, U, RMS>(b0, acc, slab, lane, ss);
-            if (i + 2 < nbatch)
-                load_batch<NT, RG, WAVES, U, RMS>(b0, wbase, abase, gbase, kt + 2 * STEP);
+            load_batch<NT, RG, WAVES, U, RMS>(b0, wrsrc, wtile, lane, abase, gbase, kt + 2 * STEP, i + 2 < nbatch);
             mma_batch<NT, RG, U, RMS>(b1, acc, slab, lane, ss);
             kt += 2 * STEP;
         }
@@ -242,7 +258,7 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     }
     for (; kt < ktiles; kt += WAVES) {
         Batch<NT, RG, 1> b;
-        load_batch<NT, RG, WAVES, 1, RMS>(b, wbase, abase, gbase, kt);
+        load_batch<NT, RG, WAVES, 1, RMS>(b, wrsrc, wtile, lane, abase, gbase, kt, true);
         mma_batch<NT, RG, 1, RMS>(b, acc, slab, lane, ss);
     }
 
@@ -322,6 +338,7 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
             }
         }
     }
+#endif
 }
 
 struct SmallMConfig {
@@ -429,6 +446,10 @@ SmallMConfig pick_small_m(int M, int N, int K, int epi, bool rms)
 
 int run_small_m(const GemmArgs &a)
 {
+    // the kernel addresses the packed weights through one buffer resource with 32-bit offsets
+    if ((size_t)a.K * a.N >= (1ull << 31))
+        return eet::fail(EET_ERR_UNSUPPORTED_SHAPE, "eet_gemm_w8a16: K x N = %d x %d exceeds the 2 GiB weight limit",
+                         a.K, a.N);
     const SmallMConfig cfg = pick_small_m(a.M, a.N, a.K, a.epi, a.rms_gamma != nullptr);
     if (a.M <= 8)
         return dispatch_small_m<1>(cfg, a);

@@ -58,9 +58,24 @@ def lib():
     return _lib
 
 
+# EET_HIP_DEBUG_SYNC=1: wait for the GPU after every library call and report a
+# failure of its kernels under that call's name -- the reference's _DEBUG_MODE_
+# build (cudaDeviceSynchronize + cudaGetLastError after each launch,
+# csrc/op/common.hpp:12, csrc/op/llama_mmha.cpp:282-285).
+DEBUG_SYNC = os.environ.get("EET_HIP_DEBUG_SYNC", "0") not in ("", "0")
+
+
 def check(status, what=""):
     """Raise RuntimeError (what the reference's pybind layer turns its
     std::runtime_error into) when a C-ABI call returned non-zero."""
     if status != 0:
         msg = lib().eet_last_error().decode("utf-8", "replace")
         raise RuntimeError(f"[EET][ERROR] {what or 'libeet_hip'}: {msg} (status {status})")
+    if DEBUG_SYNC:
+        import torch
+        if not torch.cuda.is_available():
+            return
+        try:
+            torch.cuda.synchronize()
+        except RuntimeError as e:
+            raise RuntimeError(f"[EET][ERROR] {what or 'libeet_hip'}: kernel failed: {e}") from e

@@ -2,7 +2,8 @@
 //
 // Replaces fastertransformer::gemm_fp16_int_bias_act<uint8_t>
 // (3rdparty/cutlass_kernels/fpA_intB_gemm.cu:35-62) as EET calls it: no bias,
-// no activation, no split-K workspace (csrc/op/llama_mmha.cpp:313-337).
+// no activation (csrc/op/llama_mmha.cpp:313-337).  EET never passes the split-k
+// workspace; here it is optional and used for M in the tens to hundreds.
 //
 // Weights arrive in the gfx950 layout written by eet_pack_gfx950: 1 KiB tiles
 // of 16 output channels x 64 input features, tile order [n_tile][k_tile], lane

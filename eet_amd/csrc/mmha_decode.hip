@@ -41,6 +41,13 @@ __device__ __forceinline__ float dot8(const u32x4 &a, const u32x4 &b)
     return s;
 }
 
+// A row of DH halves is DH/8 slices of 16 bytes, one per lane; the lanes of a row
+// form a group of lanes_per_row(DH) (a power of two, so that the group sum is a
+// butterfly): for DH = 96 four of the sixteen lanes of a group hold no slice, ask
+// out of range (zeros, no memory touched) and add nothing.
+constexpr int slices_per_row(int dh) { return dh / 8; }
+constexpr int lanes_per_row(int dh) { return dh == 96 ? 16 : dh / 8; }
+
 template <int WIDTH>
 __device__ __forceinline__ float group_sum(float v)
 {
@@ -59,8 +66,7 @@ template <int DH>
 __device__ __forceinline__ u32x4 rotate8(const u32x4 &x, const u32x4 &y, int sub, const float (&cs)[8],
                                          const float (&sn)[8])
 {
-    constexpr int LPR = DH / 8;
-    const bool lower = sub < LPR / 2;
+    const bool lower = sub < slices_per_row(DH) / 2;
     const half8 hx = __builtin_bit_cast(half8, x), hy = __builtin_bit_cast(half8, y);
     half8 o;
 #pragma unroll
@@ -71,7 +77,7 @@ __device__ __forceinline__ u32x4 rotate8(const u32x4 &x, const u32x4 &y, int sub
     return __builtin_bit_cast(u32x4, o);
 }
 
-// DH: head size.  LPR = DH/8 lanes cover one row with one 16-byte load each.
+// DH: head size.  The DH/8 slices of a row are covered by one 16-byte load per lane.
 // One query per (b, h) attends rows [0, step); grid = (B*H, nsplit).
 template <int DH, int UN, int THREADS>
 __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
@@ -80,8 +86,9 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
     const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, float *__restrict__ partial, int H,
     int step, int T_cap, int nsplit, float scale, const float *__restrict__ rope_row)
 {
-    constexpr int LPR = DH / 8;            // lanes per row
-    constexpr int RPB = THREADS / LPR;    // row streams of the block (one per group of LPR lanes)
+    constexpr int LPR = lanes_per_row(DH);   // lanes per row
+    constexpr int NS = slices_per_row(DH);   // of which this many hold a slice
+    constexpr int RPB = THREADS / LPR;       // row streams of the block (one per group of LPR lanes)
     __shared__ float accs[RPB][DH + 1];
     __shared__ float stream_m[RPB], stream_l[RPB];
 
@@ -92,6 +99,9 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
     const int tid = threadIdx.x;
     const int sub = tid % LPR;   // which 8-element slice of the row
     const int rs = tid / LPR;    // which row stream
+    const bool holds = sub < NS;                         // false only for the idle lanes of DH = 96
+    const unsigned idle = holds ? 0u : 0x80000000u;      // or-ed into buffer offsets: out of range
+    const int pair = sub < NS / 2 ? sub + NS / 2 : sub - NS / 2;   // the slice DH/2 away (rotary partner)
 
     const size_t qoff = qkv_stride ? (size_t)b * qkv_stride + (size_t)h * DH : (size_t)bh * DH;
     const size_t coff = (size_t)bh * DH;
@@ -132,16 +142,19 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
         const __amdgpu_buffer_rsrc_t rpr = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<float *>(rope_row ? rope_row : reinterpret_cast<const float *>(q)), 0,
             rope_row ? (unsigned)(DH * 4) : 0u, 0x00020000);
-        const int i0 = (sub % (LPR / 2)) * 8;
-        knew = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(knr, sub * 16, 0, 0));
-        kpair = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(knr, (sub ^ (LPR / 2)) * 16, 0, 0));
-        vnew = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(vnr, sub * 16, 0, 0));
-        qv = *reinterpret_cast<const u32x4 *>(q + qoff + sub * 8);
-        const u32x4 c0 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, i0 * 4, 0, 0));
-        const u32x4 c1 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, i0 * 4 + 16, 0, 0));
-        const u32x4 s0 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, (DH / 2 + i0) * 4, 0, 0));
+        const __amdgpu_buffer_rsrc_t qr = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16 *>(q + qoff), 0,
+                                                                            (unsigned)(DH * 2), 0x00020000);
+        const unsigned i0 = (unsigned)(sub % (NS / 2)) * 8u;
+        knew = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(knr, (unsigned)sub * 16u | idle, 0, 0));
+        kpair = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(knr, (unsigned)pair * 16u | idle, 0, 0));
+        vnew = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(vnr, (unsigned)sub * 16u | idle, 0, 0));
+        qv = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(qr, (unsigned)sub * 16u | idle, 0, 0));
+        const u32x4 c0 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, i0 * 4u | idle, 0, 0));
+        const u32x4 c1 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, (i0 * 4u + 16u) | idle, 0, 0));
+        const u32x4 s0 =
+            __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, (DH / 2 + i0) * 4u | idle, 0, 0));
         const u32x4 s1 =
-            __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, (DH / 2 + i0) * 4 + 16, 0, 0));
+            __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rpr, ((DH / 2 + i0) * 4u + 16u) | idle, 0, 0));
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             rcs[e] = __uint_as_float(c0[e]);
@@ -171,7 +184,7 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
         const_cast<_Float16 *>(alibi ? alibi + (size_t)h * alibi_ld + t0 : q), 0, alibi ? (unsigned)n * 2u : 0u,
         0x00020000);
     constexpr int kStream = 2;  // aux bits of a buffer load: non-temporal (every row is read exactly once)
-    auto row_off = [&](int i) { return (unsigned)((rs + i * RPB) * (DH * 2) + sub * 16); };
+    auto row_off = [&](int i) { return (unsigned)((rs + i * RPB) * (DH * 2) + sub * 16) | idle; };
     // Slot u is consumed first and refilled afterwards, so a slot's registers are
     // never live twice and the compiler keeps every slot in place: with the refill
     // ahead of the use it moved freshly requested registers at the end of each pass,
@@ -196,16 +209,17 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
     {
         const u32x4 krot = rotate8<DH>(knew, kpair, sub, rcs, rsn);
         u32x4 qy;
-        qy.x = __shfl_xor(qv.x, LPR / 2, 64);
-        qy.y = __shfl_xor(qv.y, LPR / 2, 64);
-        qy.z = __shfl_xor(qv.z, LPR / 2, 64);
-        qy.w = __shfl_xor(qv.w, LPR / 2, 64);
+        const int from = (int)(tid & 63) + pair - sub;   // the lane of this group that holds the partner slice
+        qy.x = __shfl(qv.x, from, 64);
+        qy.y = __shfl(qv.y, from, 64);
+        qy.z = __shfl(qv.z, from, 64);
+        qy.w = __shfl(qv.w, from, 64);
         const u32x4 qrot = rotate8<DH>(qv, qy, sub, rcs, rsn);
         if (rope_row != nullptr) {
             knew = krot;
             qv = qrot;
         }
-        if (append && rs == 0) {
+        if (append && rs == 0 && holds) {
             *reinterpret_cast<u32x4 *>(kc + (size_t)(step - 1) * DH + sub * 8) = knew;
             *reinterpret_cast<u32x4 *>(vc + (size_t)(step - 1) * DH + sub * 8) = vnew;
         }
@@ -247,9 +261,11 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
 #endif
 
     // Merge the RPB streams of the workgroup.
+    if (holds) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
-        accs[rs][sub * 8 + e] = acc[e];
+        for (int e = 0; e < 8; ++e)
+            accs[rs][sub * 8 + e] = acc[e];
+    }
     if (sub == 0) {
         stream_m[rs] = m_run;
         stream_l[rs] = l_run;
@@ -332,9 +348,9 @@ Plan pick_plan(int BH, int dh, int step)
         p.nsplit = forced_ns;
     if (forced_threads == 256 || forced_threads == 512 || forced_threads == 1024)
         p.threads = forced_threads;
-    else if (step / p.nsplit / (p.threads / (dh / 8)) < 8)
+    else if (step / p.nsplit / (p.threads / lanes_per_row(dh)) < 8)
         p.threads = 256;
-    const int rows_per_stream = step / p.nsplit / (p.threads / (dh / 8));
+    const int rows_per_stream = step / p.nsplit / (p.threads / lanes_per_row(dh));
     p.ring = rows_per_stream < 64 ? 2 : 4;
     if (forced_ring == 2 || forced_ring == 4 || forced_ring == 8)
         p.ring = forced_ring;
@@ -430,8 +446,8 @@ extern "C" int eet_mmha_decode(const void *q, const void *k, const void *v, long
                 "eet_mmha_decode: bad sizes B=%d H=%d step=%d T_cap=%d", B, H, step, T_cap);
     EET_REQUIRE(step <= T_cap, EET_ERR_INVALID_ARGUMENT, "eet_mmha_decode: step %d exceeds the cache capacity %d",
                 step, T_cap);
-    EET_REQUIRE(dh == 32 || dh == 64 || dh == 128, EET_ERR_UNSUPPORTED_SHAPE,
-                "eet_mmha_decode: head size %d not supported (32, 64, 128)", dh);
+    EET_REQUIRE(dh == 32 || dh == 64 || dh == 96 || dh == 128, EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_mmha_decode: head size %d not supported (32, 64, 96, 128)", dh);
     EET_REQUIRE(qkv_stride >= 0 && qkv_stride % 8 == 0, EET_ERR_INVALID_ARGUMENT,
                 "eet_mmha_decode: qkv_stride must be a non-negative multiple of 8");
     EET_REQUIRE(rope_cos_sin == nullptr || k != nullptr, EET_ERR_INVALID_ARGUMENT,
@@ -447,6 +463,9 @@ extern "C" int eet_mmha_decode(const void *q, const void *k, const void *v, long
                               ns, rope_cos_sin, st);
         case 64:
             return launch<64>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, workspace,
+                              ns, rope_cos_sin, st);
+        case 96:
+            return launch<96>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, workspace,
                               ns, rope_cos_sin, st);
         default:
             return launch<128>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap,

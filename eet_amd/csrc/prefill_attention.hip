@@ -319,13 +319,14 @@ extern "C" int eet_prefill_attention(const void *q, const void *k_cache, const v
     EET_REQUIRE(q && k_cache && v_cache && ctx, EET_ERR_INVALID_ARGUMENT, "eet_prefill_attention: null pointer");
     EET_REQUIRE(B > 0 && H > 0 && S > 0 && S <= T_cap, EET_ERR_INVALID_ARGUMENT,
                 "eet_prefill_attention: bad sizes B=%d H=%d S=%d T_cap=%d", B, H, S, T_cap);
-    EET_REQUIRE(dh == 32 || dh == 64 || dh == 128, EET_ERR_UNSUPPORTED_SHAPE,
-                "eet_prefill_attention: head size %d not supported (32, 64, 128)", dh);
+    EET_REQUIRE(dh == 32 || dh == 64 || dh == 96 || dh == 128, EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_prefill_attention: head size %d not supported (32, 64, 96, 128)", dh);
     EET_REQUIRE((long long)B * H <= 65535, EET_ERR_UNSUPPORTED_SHAPE, "eet_prefill_attention: B*H too large");
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (dh) {
         case 32: return launch<32>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
         case 64: return launch<64>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
+        case 96: return launch<96>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
         default: return launch<128>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
     }
 }

@@ -195,8 +195,8 @@ class _MmhaInt8:
             self.dh, self.inner = desc.hidden_units // H, desc.hidden_units
         else:
             self.dh, self.inner = desc.d_kv, desc.d_kv * H
-        if self.dh not in (32, 64, 128):
-            raise RuntimeError(f"[EET][ERROR] {self._name}: head size {self.dh} not supported (32, 64, 128)")
+        if self.dh not in (32, 64, 96, 128):
+            raise RuntimeError(f"[EET][ERROR] {self._name}: head size {self.dh} not supported (32, 64, 96, 128)")
         hidden = desc.hidden_units
         _check_weight("QKV_weights", QKV_weights, hidden, 3 * self.inner, desc.device)
         _check_weight("Output_weights", Output_weights, self.inner, hidden, desc.device)

@@ -139,6 +139,7 @@ int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, 
                          size_t workspace_bytes, void *stream);
 
 /* Masked multi-head decode attention for one new token per sequence.
+ *   dh        32, 64, 96 or 128, the head sizes the reference instantiates
  *   q, k, v   [B][H][dh] half; with qkv_stride != 0 they are rows of a fused
  *             buffer: element (b, h, d) at base[b * qkv_stride + h * dh + d]
  *   k_cache, v_cache  [B_cap][H][T_cap][dh] half; the new k, v are appended at

@@ -66,7 +66,7 @@ def test_device_entry_points_validate_before_launch():
     assert need >= 2 * 64 * 4096 * 4 and need % (64 * 4096 * 4) == 0
     assert L.eet_gemm_w8a16_workspace(64, 4100, 11008, 0) == 0                # not a shape the GEMM accepts
     assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 128, 9, 8, None, None, 0, None) == -1  # step > cap
-    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 96, 1, 8, None, None, 0, None) == -2   # head size
+    assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 80, 1, 8, None, None, 0, None) == -2   # head size
     assert L.eet_mmha_decode(p, p, None, 0, p, p, p, None, None, 1, 1, 128, 1, 8, None, None, 0, None) == -1     # k without v
     assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 1, 128, 1, 8, p, None, 0, None) == -1  # rotary without k
     assert L.eet_mmha_decode_workspace(8, 32, 128, 1100) == 0     # one workgroup per (b, h): no partial results
@@ -88,7 +88,7 @@ def test_device_entry_points_validate_before_launch():
     assert L.eet_qkv_split(p, p, p, p, 1, 4, 1, 128, 1, -1, 6, 8, None) == -1  # rows past the cache end
     assert L.eet_swiglu(p, p, 1, 12, None) == -2
     assert L.eet_residual_add(p, None, 1, 16, None) == -1
-    assert L.eet_prefill_attention(p, p, p, p, None, None, 1, 1, 4096, 96, 4096, None) == -2
+    assert L.eet_prefill_attention(p, p, p, p, None, None, 1, 1, 4096, 80, 4096, None) == -2
 
 
 def test_python_api_errors():

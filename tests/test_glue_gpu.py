@@ -24,7 +24,7 @@ def test_rmsnorm(gpu, M, N):
 
 @pytest.mark.parametrize("B,S,H,dh,rope,ts,t0", [(2, 5, 4, 128, 1, -1, 0), (3, 1, 4, 128, 1, 1030, 1030),
                                                    (2, 7, 5, 64, 0, -1, 0), (1, 1, 2, 32, 1, 17, 17),
-                                                   (2, 1, 40, 128, 0, 9, 9)])
+                                                   (2, 1, 40, 128, 0, 9, 9), (2, 6, 3, 96, 1, -1, 0)])
 def test_qkv_split(gpu, B, S, H, dh, rope, ts, t0):
     g = torch.Generator().manual_seed(B + S + H)
     cap = t0 + S + 3
@@ -67,7 +67,8 @@ def test_swiglu_and_residual(gpu):
                                                        (1, 4, 130, 128, False, True), (2, 2, 33, 32, True, True),
                                                        (1, 1, 1, 128, False, False), (2, 2, 64, 128, False, False),
                                                        (2, 3, 300, 128, True, False), (1, 2, 257, 64, True, True),
-                                                       (1, 2, 1024, 128, False, False), (1, 1, 2500, 128, False, True)])
+                                                       (1, 2, 1024, 128, False, False), (1, 1, 2500, 128, False, True),
+                                                       (2, 3, 200, 96, True, False), (1, 2, 77, 96, False, True)])
 def test_prefill_attention(gpu, B, H, S, dh, use_pad, use_alibi):
     g = torch.Generator().manual_seed(S)
     cap = S + 5

@@ -18,8 +18,8 @@ pytestmark = pytest.mark.gpu
 RT, AT = 2e-2, 4e-3
 
 
-def tiny_cfg(alibi=False, layers=2):
-    return D.DecoderConfig(num_layers=layers, hidden=256, heads=4, d_ff=704, vocab=512, eps=1e-6, alibi=alibi,
+def tiny_cfg(alibi=False, layers=2, hidden=256):
+    return D.DecoderConfig(num_layers=layers, hidden=hidden, heads=4, d_ff=704, vocab=512, eps=1e-6, alibi=alibi,
                            max_batch=3, max_prompt=12, max_full_seq=24)
 
 
@@ -39,9 +39,9 @@ def oracle_decoder(cfg, sd, raw):
                            sd["lm_head.weight"].numpy(), cfg.eps, n_head=cfg.heads, alibi=cfg.alibi)
 
 
-@pytest.mark.parametrize("alibi", [False, True])
-def test_single_layer_ops(gpu, alibi):
-    cfg = tiny_cfg(alibi, layers=1)
+@pytest.mark.parametrize("alibi,hidden", [(False, 256), (True, 256), (False, 384), (True, 384)])   # head size 64, 96
+def test_single_layer_ops(gpu, alibi, hidden):
+    cfg = tiny_cfg(alibi, layers=1, hidden=hidden)
     sd, raw = D.random_state_dict(cfg, seed=5)
     model = D.Int8Decoder(cfg, sd, device="cuda:0")
     ref = oracle_decoder(cfg, sd, raw)

@@ -32,6 +32,9 @@ CASES = [
     (8, 32, 128, 1025, 1153, False, False),     # BASELINE config 4, first decode step
     (8, 32, 128, 1152, 1153, False, False),     # config 4, last decode step
     (4, 40, 128, 2304, 2305, False, True),      # config 5 shape at reduced batch
+    (2, 3, 96, 1, 8, False, False),             # head size 96: 12 of the 16 lanes of a row group hold a slice
+    (2, 5, 96, 413, 420, True, True),
+    (1, 32, 96, 2100, 2100, True, False),
 ]
 
 
@@ -59,7 +62,8 @@ def test_every_launch_shape(gpu, monkeypatch, threads, ring, nsplit):
     monkeypatch.setenv("EET_MMHA_UNROLL", str(ring))
     monkeypatch.setenv("EET_MMHA_NSPLIT", str(nsplit))
     for (B, H, dh, step, use_pad, use_alibi) in [(2, 3, 128, 333, True, False), (2, 2, 64, 1207, False, True),
-                                                 (1, 2, 32, 45, True, True), (3, 2, 128, 3, False, False)]:
+                                                 (1, 2, 32, 45, True, True), (3, 2, 128, 3, False, False),
+                                                 (2, 2, 96, 290, True, True)]:
         cap = step + 3
         q, k, v, kc, vc, pad, alibi = case(B, H, dh, step, cap, step + threads, use_pad, use_alibi)
         kcn, vcn = kc.numpy().copy(), vc.numpy().copy()
@@ -113,7 +117,7 @@ def test_everything_padded_gives_zeros(gpu):
     assert not ctx[0].any() and ctx[1].any()
 
 
-@pytest.mark.parametrize("dh,step", [(128, 1), (128, 77), (64, 300), (32, 40), (128, 1100)])
+@pytest.mark.parametrize("dh,step", [(128, 1), (128, 77), (64, 300), (32, 40), (128, 1100), (96, 1), (96, 530)])
 def test_fused_rotary(gpu, dh, step):
     """q and the appended k rotated inside the kernel == rotating them first (oracle) and then attending."""
     from eet_amd._lib import check, lib

@@ -72,7 +72,7 @@ def _attn_cases(n, seed):
     rng = np.random.default_rng(seed)
     cases = []
     for i in range(n):
-        dh = [32, 64, 128][int(rng.integers(0, 3))]
+        dh = [32, 64, 96, 128][int(rng.integers(0, 4))]
         B, H = int(rng.integers(1, 6)), int(rng.integers(1, 9))
         step = int(rng.integers(1, [40, 400, 1500, 4000][i % 4]))
         cases.append((B, H, dh, step, step + int(rng.integers(0, 9)), bool(rng.integers(0, 2)), bool(rng.integers(0, 2)),

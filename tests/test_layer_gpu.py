@@ -250,3 +250,23 @@ def test_left_padded_batch(gpu, alibi):
         logits = ref.step(nxt[:, None], False, pad_np)
         got = model.logits(torch.from_numpy(nxt)[:, None].to(gpu), False, mask.to(gpu)).float().cpu().numpy()[:, 0]
     assert_close(got, logits, 3e-2, 3e-2, "logits last step")
+
+
+@pytest.mark.parametrize("alibi", [False, True])
+def test_decode_with_more_than_32_sequences(gpu, alibi):
+    """40 sequences per step: past the row count of the fused decode calls, so the ops issue RMSnorm, the
+    MFMA-tile GEMMs (with the split-k workspace), attention and the residual epilogue one by one."""
+    cfg = D.DecoderConfig(num_layers=1, hidden=256, heads=4, d_ff=704, vocab=512, eps=1e-6, alibi=alibi,
+                          max_batch=40, max_prompt=6, max_full_seq=12)
+    sd, raw = D.random_state_dict(cfg, seed=11)
+    model = D.Int8Decoder(cfg, sd, device="cuda:0")
+    ref = oracle_decoder(cfg, sd, raw)
+    g = torch.Generator().manual_seed(4)
+    ids = torch.randint(0, cfg.vocab, (40, 5), generator=g)
+    logits = ref.step(ids.numpy(), True)
+    got = model.logits(ids.to(gpu), True).float().cpu().numpy()[:, 0]
+    for t in range(3):
+        assert_close(got, logits, 3e-2, 3e-2, f"logits step {t}")
+        nxt = logits.argmax(-1)
+        logits = ref.step(nxt[:, None], False)
+        got = model.logits(torch.from_numpy(nxt)[:, None].to(gpu), False).float().cpu().numpy()[:, 0]

@@ -266,7 +266,7 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0   # MI355X published dense fp16 MFMA peak
 
 
 def prefill_gemm_bench(torch, eet, lib, dev, iters=10):
-    """BASELINE config 3: Baichuan-13B-shaped prefill GEMMs, M = 2048 tokens, on the MFMA kernel.
+    """benchmark configuration 3: Baichuan-13B-shaped prefill GEMMs, M = 2048 tokens, on the MFMA kernel.
     Reports TFLOP/s = 2*M*N*K / t and the fraction of the fp16 MFMA peak."""
     M, hidden, d_ff = 2048, 5120, 13696
     g = torch.Generator(device=dev).manual_seed(21)
@@ -354,7 +354,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the M = 1..32 sweep")
     ap.add_argument("--baichuan", action="store_true",
-                    help="also run BASELINE config 5: Baichuan-13B-shaped decoder (40 layers, ALiBi), batch 32, "
+                    help="also run benchmark configuration 5: Baichuan-13B-shaped decoder (40 layers, ALiBi), batch 32, "
                          "prompt 2048, 256 greedy tokens (needs ~85 GB of HBM and about a minute)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 1 GiB device-to-device copies (a kernel of known traffic, for scaling "

@@ -31,7 +31,7 @@ def test_small_shapes(gpu, M, K, N):
     assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32), what=f"{M}x{K}x{N}")
 
 
-# BASELINE configs 1 and 2: LLaMA-7B decode linears at M in {1, 4, 8, 16, 32}
+# benchmark configurations 1 and 2: LLaMA-7B decode linears at M in {1, 4, 8, 16, 32}
 @pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 12288), (4096, 11008), (11008, 4096)])
 def test_llama7b_shapes(gpu, K, N):
     x, u, p, s = make(32, K, N, K + N)
@@ -43,7 +43,7 @@ def test_llama7b_shapes(gpu, K, N):
 
 
 def test_config1_sym127(gpu):
-    """BASELINE config 1 as worded: /127 scales, int8 in [-127, 127], M = 1."""
+    """benchmark configuration 1 as worded: /127 scales, int8 in [-127, 127], M = 1."""
     x, u, p, s = make(1, 4096, 4096, 1, mode="sym127")
     c = gemm(x.to(gpu), p.to(gpu), s.to(gpu), 1, 4096, 4096)
     assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32))
@@ -124,7 +124,7 @@ def test_large_m_dispatch(gpu, M, K, N, tile):
 
 
 def test_full_size_linearity(gpu):
-    """Size-independent property at a BASELINE shape: gemm(a + b) == gemm(a) + gemm(b) within fp16 rounding,
+    """Size-independent property at a benchmark shape: gemm(a + b) == gemm(a) + gemm(b) within fp16 rounding,
     and doubling the scales doubles the output exactly."""
     K, N, M = 4096, 11008, 8
     g = torch.Generator().manual_seed(11)

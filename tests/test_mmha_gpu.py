@@ -29,7 +29,7 @@ CASES = [
     (2, 2, 32, 70, 80, True, True),
     (1, 8, 128, 4096, 4100, False, False),      # past the reference's 4096-step limit? no: exactly at it
     (1, 2, 128, 5000, 5000, True, False),       # beyond it
-    (8, 32, 128, 1025, 1153, False, False),     # BASELINE config 4, first decode step
+    (8, 32, 128, 1025, 1153, False, False),     # benchmark configuration 4, first decode step
     (8, 32, 128, 1152, 1153, False, False),     # config 4, last decode step
     (4, 40, 128, 2304, 2305, False, True),      # config 5 shape at reduced batch
     (2, 3, 96, 1, 8, False, False),             # head size 96: 12 of the 16 lanes of a row group hold a slice
@@ -139,7 +139,7 @@ def test_fused_rotary(gpu, dh, step):
     assert np.array_equal(vcd.cpu().numpy(), vcn)
 
 
-@pytest.mark.parametrize("B,H,step,cap,use_alibi", [(8, 32, 1152, 1153, False),      # BASELINE config 4, full size
+@pytest.mark.parametrize("B,H,step,cap,use_alibi", [(8, 32, 1152, 1153, False),      # benchmark configuration 4, full size
                                                     (32, 40, 2304, 2305, True)])     # config 5, full size
 def test_full_size_uniform_keys(gpu, B, H, step, cap, use_alibi):
     """Size-independent property at the full benchmark shapes: when every cached key of a head equals the new

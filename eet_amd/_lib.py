@@ -16,6 +16,7 @@ _vp, _i, _sz, _f, _l = _c.c_void_p, _c.c_int, _c.c_size_t, _c.c_float, _c.c_long
 SIGNATURES = {
     "eet_last_error": (_c.c_char_p, []),
     "eet_packed_layout_version": (_i, []),
+    "eet_set_tuning": (_i, [_c.c_char_p, _c.c_char_p]),
     "eet_quantize_int8": (_i, [_vp, _i, _sz, _sz, _i, _vp, _vp]),
     "eet_pack_gfx950": (_i, [_vp, _sz, _sz, _vp]),
     "eet_unpack_gfx950": (_i, [_vp, _sz, _sz, _vp]),

@@ -14,6 +14,15 @@
 
 #include "common.h"
 
+namespace {
+// do the byte ranges [a, a + an) and [b, b + bn) share a byte?
+bool overlaps(const void *a, size_t an, const void *b, size_t bn)
+{
+    const uintptr_t x = reinterpret_cast<uintptr_t>(a), y = reinterpret_cast<uintptr_t>(b);
+    return x < y + bn && y < x + an;
+}
+}  // namespace
+
 extern "C" size_t eet_mmha_int8_decode_workspace(int B, int H, int dh, int step)
 {
     return eet_mmha_decode_workspace(B, H, dh, step);
@@ -30,9 +39,19 @@ extern "C" int eet_mmha_int8_decode(const void *x, const void *rms_gamma, float 
     EET_REQUIRE(B > 0 && B <= 32 && H > 0 && dh > 0 && hidden > 0, EET_ERR_UNSUPPORTED_SHAPE,
                 "eet_mmha_int8_decode: B=%d must be 1..32 (one token per sequence), H=%d dh=%d hidden=%d", B, H, dh,
                 hidden);
-    EET_REQUIRE(out != x, EET_ERR_INVALID_ARGUMENT,
-                "eet_mmha_int8_decode: out must not alias x (x is the residual of the last launch)");
     const int inner = H * dh;
+    {
+        // x is read by the first launch and again, as the residual, by the last; every
+        // buffer written in between must stay clear of it and of what the launch that
+        // writes it reads
+        const size_t xb = (size_t)B * hidden * 2, qb = (size_t)B * 3 * inner * 2, cb = (size_t)B * inner * 2;
+        EET_REQUIRE(!overlaps(out, xb, x, xb) && !overlaps(qkv_buf, qb, x, xb) && !overlaps(ctx_buf, cb, x, xb),
+                    EET_ERR_INVALID_ARGUMENT,
+                    "eet_mmha_int8_decode: out, qkv_buf and ctx_buf must not overlap x (x is the residual of the "
+                    "last launch)");
+        EET_REQUIRE(!overlaps(ctx_buf, cb, qkv_buf, qb) && !overlaps(out, xb, ctx_buf, cb), EET_ERR_INVALID_ARGUMENT,
+                    "eet_mmha_int8_decode: ctx_buf must not overlap qkv_buf, nor out ctx_buf");
+    }
     // RMSnorm + QKV projection (llama_mmha.cpp:222-227)
     if (int rc = eet_gemm_w8a16_fused(x, qkv_w, qkv_scale, qkv_buf, B, 3 * inner, hidden, EET_EPILOGUE_NONE, nullptr,
                                       rms_gamma, rms_eps, nullptr, 0, stream))
@@ -55,7 +74,11 @@ extern "C" int eet_gated_ffn_int8_decode(const void *x, const void *rms_gamma, f
     EET_REQUIRE(B > 0 && B <= 32 && hidden > 0 && d_ff > 0, EET_ERR_UNSUPPORTED_SHAPE,
                 "eet_gated_ffn_int8_decode: B=%d must be 1..32 (one token per sequence), hidden=%d d_ff=%d", B, hidden,
                 d_ff);
-    EET_REQUIRE(out != x, EET_ERR_INVALID_ARGUMENT, "eet_gated_ffn_int8_decode: out must not alias x");
+    {
+        const size_t xb = (size_t)B * hidden * 2, ab = (size_t)B * d_ff * 2;
+        EET_REQUIRE(!overlaps(out, xb, x, xb) && !overlaps(act_buf, ab, x, xb) && !overlaps(out, xb, act_buf, ab),
+                    EET_ERR_INVALID_ARGUMENT, "eet_gated_ffn_int8_decode: x, act_buf and out must not overlap");
+    }
     // RMSnorm + gate and up projections + SwiGLU (gated_ffn_int8.cpp:112-120): w01 holds gate and up
     // interleaved by 16-channel tile
     if (int rc = eet_gemm_w8a16_fused(x, w01, scale01, act_buf, B, 2 * d_ff, hidden, EET_EPILOGUE_SWIGLU, nullptr,

@@ -26,9 +26,8 @@
 // more accurate and inside the 1e-2 / 1e-3 tolerance against fp32).
 #include <hip/hip_runtime.h>
 
-#include <cstdlib>
-
 #include "gemm_common.h"
+#include "tuning.h"
 
 using namespace eet;
 
@@ -414,12 +413,6 @@ int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a)
 // wavefronts when there are few workgroups (more loads in flight per CU).
 SmallMConfig pick_small_m(int M, int N, int K, int epi, bool rms)
 {
-    const char *env = std::getenv("EET_GEMM_SMALL_M_CONFIG");  // "nt,waves,u": tuning override
-    if (env) {
-        SmallMConfig c{1, 8, 4};
-        if (sscanf(env, "%d,%d,%d", &c.nt, &c.waves, &c.u) == 3 && (epi != kEpiSwiglu || c.nt % 2 == 0))
-            return c;
-    }
     const int ntiles = N / 16;
     (void)K;
     int best_nt = 0;
@@ -451,12 +444,19 @@ int run_small_m(const GemmArgs &a)
     if ((size_t)a.K * a.N >= (1ull << 31))
         return eet::fail(EET_ERR_UNSUPPORTED_SHAPE, "eet_gemm_w8a16: K x N = %d x %d exceeds the 2 GiB weight limit",
                          a.K, a.N);
-    const SmallMConfig cfg = pick_small_m(a.M, a.N, a.K, a.epi, a.rms_gamma != nullptr);
-    if (a.M <= 8)
-        return dispatch_small_m<1>(cfg, a);
-    if (a.M <= 16)
-        return dispatch_small_m<2>(cfg, a);
-    return dispatch_small_m<4>(cfg, a);
+    auto dispatch = [&](SmallMConfig cfg) {
+        if (a.M <= 8)
+            return dispatch_small_m<1>(cfg, a);
+        if (a.M <= 16)
+            return dispatch_small_m<2>(cfg, a);
+        return dispatch_small_m<4>(cfg, a);
+    };
+    // a tuning override runs when such a kernel exists for this call; otherwise the table decides
+    const eet::Tuning &tune = eet::tuning();
+    if (tune.has_small_m && (a.epi != kEpiSwiglu || tune.small_m_nt % 2 == 0) &&
+        dispatch(SmallMConfig{tune.small_m_nt, tune.small_m_waves, tune.small_m_u}) == EET_OK)
+        return EET_OK;
+    return dispatch(pick_small_m(a.M, a.N, a.K, a.epi, a.rms_gamma != nullptr));
 }
 
 }  // namespace
@@ -480,7 +480,7 @@ static int run_gemm(const GemmArgs &a)
     const size_t split_bytes = eet::large_m_workspace(a.M, a.N, a.K, a.epi);
     const bool can_split = split_bytes > 0 && a.ws != nullptr && a.ws_bytes >= split_bytes &&
                            reinterpret_cast<uintptr_t>(a.ws) % 16 == 0;
-    if (takes_slabs(a.M, a.N) && !can_split && std::getenv("EET_GEMM_LARGE_M_TILE") == nullptr) {
+    if (takes_slabs(a.M, a.N) && !can_split && !eet::tuning().has_large_m) {
         const int n_out = (a.epi == kEpiSwiglu) ? a.N / 2 : a.N;
         for (int m0 = 0; m0 < a.M; m0 += 32) {
             GemmArgs s = a;

@@ -32,9 +32,8 @@
 // 128 B, whole cache lines; the XOR only permutes lanes within a line), and the
 // MFMA operand read of lane (g, j) -- piece 2g+h of row j -- hits 16 distinct
 // 16-byte bank groups per 16 lanes.
-#include <cstdlib>
-
 #include "gemm_common.h"
+#include "tuning.h"
 
 using namespace eet;
 
@@ -90,8 +89,11 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
     const int nt0 = n_blk * (WNW * TN) + wave * TN;
 
     // Both operands are addressed through buffer resources: a 32-bit lane offset
-    // plus a scalar offset per tile, and reads past the end (rows >= M, n-tiles
-    // >= N/16) return zeros instead of needing clamped addresses.
+    // plus a scalar offset per tile.  The range check of a buffer load covers the
+    // lane offset only, not the scalar one: activation rows >= M are out of range
+    // by their lane offset and read as zeros; the weight tile index lives in the
+    // scalar offset, so an n-tile >= N/16 of a block that overhangs N is clamped
+    // to the last real tile (its products are never stored).
     const size_t a_bytes = (size_t)(M - m0) * K * 2;
     const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<_Float16 *>(A + (size_t)m0 * K), 0, a_bytes > 0xffffffffull ? 0xffffffffu : (unsigned)a_bytes,
@@ -102,7 +104,7 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
     unsigned wtile[TN];  // byte offset of the n-tile's first k-tile
 #pragma unroll
     for (int t = 0; t < TN; ++t)
-        wtile[t] = (unsigned)(nt0 + t) * (unsigned)ktiles * 1024u;
+        wtile[t] = (unsigned)min(nt0 + t, ntiles - 1) * (unsigned)ktiles * 1024u;
 
     // DMA source of this lane for row group rg = wave * kPerWave + i: row
     // 8*rg + lane/8, piece (lane%8) ^ swizzle.
@@ -429,14 +431,12 @@ int eet::run_large_m(const GemmArgs &a)
     LargeMConfig c = pick_large_m(a.M, a.N, a.K, a.epi, true);
     if (!fits(c.ksplit))
         c = pick_large_m(a.M, a.N, a.K, a.epi, false);
-    if (const char *env = std::getenv("EET_GEMM_LARGE_M_TILE")) {  // "tm,tn[,ksplit]": tuning override
-        LargeMConfig e = c;
-        const int got = sscanf(env, "%d,%d,%d", &e.tm, &e.tn, &e.ksplit);
-        if (got >= 2 && (a.epi != kEpiSwiglu || e.tn % 2 == 0)) {
-            if (got == 2)
-                e.ksplit = 1;
-            c = e;
-        }
+    const eet::Tuning &tune = eet::tuning();
+    if (tune.has_large_m) {  // "tm,tn[,ksplit]": runs when such a tile exists, else the table's choice stands
+        const int tm = tune.large_m_tm, tn = tune.large_m_tn;
+        const bool exists = (tm == 8 && tn == 4) || (tm == 4 && (tn == 5 || tn == 4 || tn == 2)) || (tm == 2 && tn == 2);
+        if (exists && (a.epi != kEpiSwiglu || tn % 2 == 0))
+            c = LargeMConfig{tm, tn, tune.large_m_ksplit > 0 ? tune.large_m_ksplit : 1};
         if (!fits(c.ksplit))
             c.ksplit = 1;
     }

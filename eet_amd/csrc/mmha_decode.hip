@@ -20,9 +20,9 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
-#include <cstdlib>
 
 #include "common.h"
+#include "tuning.h"
 
 namespace {
 
@@ -332,13 +332,8 @@ struct Plan {
 
 Plan pick_plan(int BH, int dh, int step)
 {
-    // tuning overrides, read on every call (a getenv is noise next to a launch)
-    auto env_int = [](const char *name) {
-        const char *e = std::getenv(name);
-        return e ? atoi(e) : 0;
-    };
-    const int forced_ns = env_int("EET_MMHA_NSPLIT"), forced_threads = env_int("EET_MMHA_THREADS");
-    const int forced_ring = env_int("EET_MMHA_UNROLL");
+    const eet::Tuning &tune = eet::tuning();
+    const int forced_ns = tune.mmha_nsplit, forced_threads = tune.mmha_threads, forced_ring = tune.mmha_ring;
     Plan p{512, 1, 4};
     const int want = (256 + BH - 1) / BH, by_rows = step / 256;
     p.nsplit = want < by_rows ? want : by_rows;
@@ -434,41 +429,59 @@ extern "C" size_t eet_mmha_decode_workspace(int B, int H, int dh, int step)
     return ns > 1 ? (size_t)B * H * ns * (dh + 2) * sizeof(float) : 0;
 }
 
+// Argument checks shared by the two entry points; fills `plan`.
+static int check_mmha_args(const char *fn, const void *q, const void *k, const void *v, long qkv_stride,
+                           const void *k_cache, const void *v_cache, const void *ctx, int B, int H, int dh, int step,
+                           int T_cap, const float *rope_cos_sin, Plan *plan)
+{
+    EET_REQUIRE(q && k_cache && v_cache && ctx, EET_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+    EET_REQUIRE((k == nullptr) == (v == nullptr), EET_ERR_INVALID_ARGUMENT,
+                "%s: k and v must both be given or both be NULL", fn);
+    EET_REQUIRE(B > 0 && H > 0 && step > 0 && T_cap > 0, EET_ERR_INVALID_ARGUMENT,
+                "%s: bad sizes B=%d H=%d step=%d T_cap=%d", fn, B, H, step, T_cap);
+    EET_REQUIRE(step <= T_cap, EET_ERR_INVALID_ARGUMENT, "%s: step %d exceeds the cache capacity %d", fn, step, T_cap);
+    EET_REQUIRE(dh == 32 || dh == 64 || dh == 96 || dh == 128, EET_ERR_UNSUPPORTED_SHAPE,
+                "%s: head size %d not supported (32, 64, 96, 128)", fn, dh);
+    EET_REQUIRE(qkv_stride >= 0 && qkv_stride % 8 == 0, EET_ERR_INVALID_ARGUMENT,
+                "%s: qkv_stride must be a non-negative multiple of 8", fn);
+    EET_REQUIRE(rope_cos_sin == nullptr || k != nullptr, EET_ERR_INVALID_ARGUMENT,
+                "%s: a rotary row needs the new k, v (it rotates q and the appended k)", fn);
+    *plan = pick_plan(B * H, dh, step);
+    return EET_OK;
+}
+
+static int run_mmha(const void *q, const void *k, const void *v, long qkv_stride, void *k_cache, void *v_cache,
+                    void *ctx, const void *alibi, const int64_t *pad, int B, int H, int dh, int step, int T_cap,
+                    const float *rope_cos_sin, void *partials, Plan plan, hipStream_t st)
+{
+    switch (dh) {
+        case 32:
+            return launch<32>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, partials,
+                              plan, rope_cos_sin, st);
+        case 64:
+            return launch<64>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, partials,
+                              plan, rope_cos_sin, st);
+        case 96:
+            return launch<96>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, partials,
+                              plan, rope_cos_sin, st);
+        default:
+            return launch<128>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, partials,
+                               plan, rope_cos_sin, st);
+    }
+}
+
 extern "C" int eet_mmha_decode(const void *q, const void *k, const void *v, long qkv_stride, void *k_cache,
                                void *v_cache, void *ctx, const void *alibi, const int64_t *pad, int B, int H,
                                int dh, int step, int T_cap, const float *rope_cos_sin, void *workspace,
                                size_t workspace_bytes, void *stream)
 {
-    EET_REQUIRE(q && k_cache && v_cache && ctx, EET_ERR_INVALID_ARGUMENT, "eet_mmha_decode: null pointer");
-    EET_REQUIRE((k == nullptr) == (v == nullptr), EET_ERR_INVALID_ARGUMENT,
-                "eet_mmha_decode: k and v must both be given or both be NULL");
-    EET_REQUIRE(B > 0 && H > 0 && step > 0 && T_cap > 0, EET_ERR_INVALID_ARGUMENT,
-                "eet_mmha_decode: bad sizes B=%d H=%d step=%d T_cap=%d", B, H, step, T_cap);
-    EET_REQUIRE(step <= T_cap, EET_ERR_INVALID_ARGUMENT, "eet_mmha_decode: step %d exceeds the cache capacity %d",
-                step, T_cap);
-    EET_REQUIRE(dh == 32 || dh == 64 || dh == 96 || dh == 128, EET_ERR_UNSUPPORTED_SHAPE,
-                "eet_mmha_decode: head size %d not supported (32, 64, 96, 128)", dh);
-    EET_REQUIRE(qkv_stride >= 0 && qkv_stride % 8 == 0, EET_ERR_INVALID_ARGUMENT,
-                "eet_mmha_decode: qkv_stride must be a non-negative multiple of 8");
-    EET_REQUIRE(rope_cos_sin == nullptr || k != nullptr, EET_ERR_INVALID_ARGUMENT,
-                "eet_mmha_decode: a rotary row needs the new k, v (it rotates q and the appended k)");
-    const Plan ns = pick_plan(B * H, dh, step);
-    const size_t need = eet_mmha_decode_workspace(B, H, dh, step);
+    Plan plan;
+    if (int rc = check_mmha_args("eet_mmha_decode", q, k, v, qkv_stride, k_cache, v_cache, ctx, B, H, dh, step,
+                                 T_cap, rope_cos_sin, &plan))
+        return rc;
+    const size_t need = plan.nsplit > 1 ? (size_t)B * H * plan.nsplit * (dh + 2) * sizeof(float) : 0;
     EET_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), EET_ERR_WORKSPACE,
                 "eet_mmha_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    switch (dh) {
-        case 32:
-            return launch<32>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, workspace,
-                              ns, rope_cos_sin, st);
-        case 64:
-            return launch<64>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, workspace,
-                              ns, rope_cos_sin, st);
-        case 96:
-            return launch<96>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, workspace,
-                              ns, rope_cos_sin, st);
-        default:
-            return launch<128>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap,
-                               workspace, ns, rope_cos_sin, st);
-    }
+    return run_mmha(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, dh, step, T_cap, rope_cos_sin,
+                    workspace, plan, static_cast<hipStream_t>(stream));
 }

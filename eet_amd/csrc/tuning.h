@@ -1,0 +1,24 @@
+// Tuning overrides of the launch-shape tables, for sweeps and for the tests that
+// run every kernel variant.  Nothing on the launch path reads the environment:
+// the overrides live in one process-wide block that is written only by
+// eet_set_tuning() and, once at library load, from the environment when
+// EET_HIP_TUNING=1 is set.  An override that names a kernel variant that does not
+// exist is ignored by the dispatcher (the table's choice runs instead).
+#pragma once
+
+namespace eet {
+
+struct Tuning {
+    // EET_GEMM_SMALL_M_CONFIG = "nt,waves,u"
+    bool has_small_m = false;
+    int small_m_nt = 0, small_m_waves = 0, small_m_u = 0;
+    // EET_GEMM_LARGE_M_TILE = "tm,tn[,ksplit]"
+    bool has_large_m = false;
+    int large_m_tm = 0, large_m_tn = 0, large_m_ksplit = 0;  // ksplit 0: not given
+    // EET_MMHA_NSPLIT, EET_MMHA_THREADS, EET_MMHA_UNROLL (0: not given)
+    int mmha_nsplit = 0, mmha_threads = 0, mmha_ring = 0;
+};
+
+const Tuning &tuning();
+
+}  // namespace eet

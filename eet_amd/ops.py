@@ -74,6 +74,31 @@ class _Workspaces:
 workspaces = _Workspaces()
 
 
+class _SpareKV:
+    """The second KV buffer of the beam-search reorder, shared by every attention op with the
+    same cache shape on a device: an op gathers into the spare pair, takes it as its cache and
+    leaves its old pair as the new spare.  The ops of a decoder run one after another on one
+    stream, so a single spare serves all layers."""
+
+    def __init__(self):
+        self._pairs = {}
+
+    def swap(self, k_cache, v_cache, gather):
+        key = (tuple(k_cache.shape), k_cache.dtype, str(k_cache.device))
+        pair = self._pairs.get(key)
+        if pair is None:
+            pair = (torch.zeros_like(k_cache), torch.zeros_like(v_cache))
+        gather(pair[0], pair[1])
+        self._pairs[key] = (k_cache, v_cache)
+        return pair
+
+    def clear(self):
+        self._pairs.clear()
+
+
+spare_kv = _SpareKV()
+
+
 # ----------------------------------------------------------------------------
 # MetaDesc
 # ----------------------------------------------------------------------------
@@ -211,7 +236,6 @@ class _MmhaInt8:
         # KV cache, private to the op (csrc/op/llama_mmha.cpp:47-48); layout [B][H][T][dh]
         self.k_cache = torch.zeros(desc.batch_size, H, self.t_cap, self.dh, dtype=torch.float16, device=dev)
         self.v_cache = torch.zeros_like(self.k_cache)
-        self._k_spare = self._v_spare = None     # second buffer of the beam-search reorder, made on first use
         self.step = 1
         self.first_batch = 0
         self.rope_table = _rope_table(self.t_cap, self.dh, dev) if self._rope else None
@@ -271,14 +295,13 @@ class _MmhaInt8:
         L = lib()
         if reorder is not None and not first_pass:
             # beam b continues from the rows of beam reorder[b] (csrc/op/llama_mmha.cpp:248-252):
-            # gather into the second cache buffer, then swap the two
-            if self._k_spare is None:
-                self._k_spare, self._v_spare = torch.zeros_like(self.k_cache), torch.zeros_like(self.v_cache)
-            check(L.eet_kv_cache_reorder(self.k_cache.data_ptr(), self.v_cache.data_ptr(), self._k_spare.data_ptr(),
-                                         self._v_spare.data_ptr(), reorder.data_ptr(), self.first_batch, H, dh,
-                                         self.step - 1, self.t_cap, _stream()), "eet_kv_cache_reorder")
-            self.k_cache, self._k_spare = self._k_spare, self.k_cache
-            self.v_cache, self._v_spare = self._v_spare, self.v_cache
+            # gather into the spare cache pair (one per cache shape, shared by all layers), then
+            # take that pair as this op's cache
+            def gather(k_dst, v_dst):
+                check(L.eet_kv_cache_reorder(self.k_cache.data_ptr(), self.v_cache.data_ptr(), k_dst.data_ptr(),
+                                             v_dst.data_ptr(), reorder.data_ptr(), self.first_batch, H, dh,
+                                             self.step - 1, self.t_cap, _stream()), "eet_kv_cache_reorder")
+            self.k_cache, self.v_cache = spare_kv.swap(self.k_cache, self.v_cache, gather)
         f16 = torch.float16
         xn = workspaces.get("layernorm", desc.batch_size * max(desc.max_seq_len, 1) * hidden, f16, dev)
         qkv = workspaces.get("qkv", desc.batch_size * max(desc.max_seq_len, 1) * 3 * self.inner, f16, dev)
@@ -391,12 +414,12 @@ class GatedFeedForwardNetworkInt8:
         _check_vec("Intermediate_1_scale", Intermediate_1_scale, self.d_ff)
         _check_vec("Output_scale", Output_scale, hidden)
         _check_vec("layernorm_weights", layernorm_weights, hidden)
-        self.w0, self.s0, self.w1, self.s1, self.w2, self.s2, self.gamma = (
-            Intermediate_0_weights, Intermediate_0_scale, Intermediate_1_weights, Intermediate_1_scale,
-            Output_weights, Output_scale, layernorm_weights)
+        self.w2, self.s2, self.gamma = Output_weights, Output_scale, layernorm_weights
         self.cache_name = ffn_cache_name
-        # gate and up merged tile by tile so that one launch computes both and applies SwiGLU
-        self.w01, self.s01 = interleave_gate_up(self.w0, self.s0, self.w1, self.s1)
+        # gate and up merged tile by tile so that one launch computes both and applies SwiGLU;
+        # the op keeps only the merged copy (the caller's separate tensors can be freed)
+        self.w01, self.s01 = interleave_gate_up(Intermediate_0_weights, Intermediate_0_scale,
+                                                Intermediate_1_weights, Intermediate_1_scale)
 
     def forward(self, input, pre_layernorm, add_residual):
         with _StreamScope():
@@ -506,20 +529,26 @@ def pack_weights_torch(q):
     return t.permute(3, 0, 1, 4, 2).contiguous().view(torch.int8).view(K, N)
 
 
+def _round_half_away(r):
+    """C round(): r - trunc(r) is exact in binary floating point, so unlike
+    floor(|r| + 0.5) this never rounds twice (0.49999997f stays 0)."""
+    t = torch.trunc(r)
+    return t + torch.where((r - t).abs() >= 0.5, torch.sign(r), torch.zeros_like(r))
+
+
 def quant_weights_torch(w, mode="ref128"):
-    """The quantiser as torch ops on w's device (fp32 math, same rules as
-    eet_quantize_int8): returns (unprocessed int8 [K, N], scales in w's dtype)."""
+    """The quantiser as torch ops on w's device, bit-identical to
+    eet_quantize_int8 (fp32 math, one correctly rounded operation per step):
+    returns (unprocessed int8 [K, N], scales in w's dtype)."""
     w32 = w.float()
     amax = w32.abs().amax(0)
     if mode == "ref128":
         s32 = amax * (1.0 / 128.0)
-        r = w32 / s32
-        r = torch.where(r >= 0, torch.floor(r.abs() + 0.5), -torch.floor(r.abs() + 0.5))
+        r = _round_half_away(w32 / s32)
         r = torch.where(torch.isnan(r), torch.full_like(r, 127.0), r).clamp(-128, 127)
     else:
         s32 = amax / 127.0
-        r = w32 / s32
-        r = torch.where(r >= 0, torch.floor(r.abs() + 0.5), -torch.floor(r.abs() + 0.5))
+        r = _round_half_away(w32 / s32)
         r = torch.where(torch.isnan(r), torch.zeros_like(r), r).clamp(-127, 127)
     return r.to(torch.int8), s32.to(w.dtype)
 

@@ -47,6 +47,17 @@ const char *eet_last_error(void);
 /* Version tag of the packed weight layout produced by eet_pack_gfx950. */
 int eet_packed_layout_version(void);
 
+/* Overrides one of the library's launch-shape tables, for sweeps and for tests
+ * that run every kernel variant; value NULL or "" restores the table.  Keys:
+ *   EET_GEMM_SMALL_M_CONFIG "nt,waves,u"       EET_GEMM_LARGE_M_TILE "tm,tn[,ksplit]"
+ *   EET_MMHA_NSPLIT / EET_MMHA_THREADS / EET_MMHA_UNROLL "n"
+ * An override naming a kernel variant that does not exist is ignored.  The same
+ * keys are read from the environment once, at load, when EET_HIP_TUNING=1; no
+ * launch reads the environment (the reference queries occupancy and runs its
+ * heuristic on every call: fpA_intB_gemm_template.h:460-491).  Process-wide and
+ * not synchronised: call it while no launch of this library is being issued. */
+int eet_set_tuning(const char *name, const char *value);
+
 /* ------------------------------------------------------------------------
  * Offline weight packer (host CPU, no GPU needed).
  * ---------------------------------------------------------------------- */

@@ -21,9 +21,17 @@ checkout).  How each function is pinned:
   decode_attention       step=1 => v/(1+1e-6), uniform keys => mean(V),
                          brute-force softmax, padded prefix has zero weight
   alibi_slopes / mask    closed form for n=40 and powers of two
-  layer / decoder        composition of the above (no independent pin:
-                         the reference holds no test, fixture or golden
-                         vector for any function on this path)
+  quantize_sym127        scalar brute force; closed-form scale; extremes at +-127
+  layer / decoder        an independently written float64 model in the Hugging
+                         Face formulation without a KV cache
+                         (tests/hf_formulation.py), with planted-mistake
+                         controls; zero-projection identity; one-token closed
+                         form; incremental call == last row of a longer prefill
+                         (tests/test_oracle_composition.py)
+
+The reference itself holds no test, fixture or golden vector for any function
+on this path, so every pin above is one the mathematics or the published model
+definitions fix.
 
 The reference's own build of the quantiser needs <cuda_runtime.h> and the
 cutlass headers, which this image lacks, so no oracle/_ref build exists.

@@ -33,3 +33,17 @@ def gpu():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def tuning():
+    """Sets launch-shape overrides through eet_set_tuning for one test and clears them afterwards."""
+    from eet_amd._lib import check, lib
+    used = []
+
+    def set_(name, value):
+        used.append(name)
+        check(lib().eet_set_tuning(name.encode(), str(value).encode()), "eet_set_tuning")
+    yield set_
+    for name in used:
+        lib().eet_set_tuning(name.encode(), None)

@@ -100,10 +100,10 @@ LARGE_M_TILES = ["8,4", "4,5", "4,4", "4,2", "2,2"]   # m-tiles, n-tiles per wav
 
 
 @pytest.mark.parametrize("tile", LARGE_M_TILES)
-def test_large_m_tiles(gpu, monkeypatch, tile):
+def test_large_m_tiles(gpu, tuning, tile):
     """Every large-M kernel variant (selected with the tuning override), on ragged M / N edges and on
     k-loops of 1..9 tiles (prologue, unrolled body and tail of the software pipeline)."""
-    monkeypatch.setenv("EET_GEMM_LARGE_M_TILE", tile)
+    tuning("EET_GEMM_LARGE_M_TILE", tile)
     for (M, K, N) in [(129, 64, 48), (300, 128, 272), (257, 192, 720), (200, 256, 336), (512, 320, 256),
                       (130, 448, 64), (333, 576, 1040)]:
         x, u, p, s = make(M, K, N, M + K + N)
@@ -180,11 +180,11 @@ def test_swiglu_epilogue(gpu, M, K, F):
 
 
 @pytest.mark.parametrize("tile", LARGE_M_TILES)
-def test_large_m_tile_epilogues(gpu, monkeypatch, tile):
+def test_large_m_tile_epilogues(gpu, tuning, tile):
     """Residual and SwiGLU epilogues of every large-M kernel variant (5 n-tiles per wavefront cannot
     pair gate / up tiles: there the override is ignored for SwiGLU and the dispatcher's own choice runs)."""
     from eet_amd.ops import interleave_gate_up
-    monkeypatch.setenv("EET_GEMM_LARGE_M_TILE", tile)
+    tuning("EET_GEMM_LARGE_M_TILE", tile)
     M, K, N = 270, 320, 592
     x, u, p, s = make(M, K, N, 5)
     res = torch.randn(M, N, generator=torch.Generator().manual_seed(M)).half()
@@ -211,12 +211,12 @@ SPLIT_K = ["2,2,2", "2,2,3", "2,2,8", "4,2,4", "4,4,2", "8,4,5"]   # m-tiles, n-
 
 @pytest.mark.parametrize("cfg", SPLIT_K)
 @pytest.mark.parametrize("M,K,N", [(70, 1216, 400), (33, 4096, 1024), (161, 640, 528)])
-def test_split_k(gpu, monkeypatch, cfg, M, K, N):
+def test_split_k(gpu, tuning, cfg, M, K, N):
     """Every tile with its k range shared by several workgroups (uneven shares, ragged rows and channels,
     one k-tile per part at K = 640 with 8 parts) + the second kernel that adds the fp32 parts, for all three
     epilogues, against the fp32 oracle; without the workspace the same call runs in a single pass."""
     from eet_amd.ops import interleave_gate_up
-    monkeypatch.setenv("EET_GEMM_LARGE_M_TILE", cfg)
+    tuning("EET_GEMM_LARGE_M_TILE", cfg)
     ws = 8 * M * max(N, 1024) * 4
     x, u, p, s = make(M, K, N, 11)
     res = torch.randn(M, N, generator=torch.Generator().manual_seed(M)).half()

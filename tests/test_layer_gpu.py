@@ -270,3 +270,99 @@ def test_decode_with_more_than_32_sequences(gpu, alibi):
         nxt = logits.argmax(-1)
         logits = ref.step(nxt[:, None], False)
         got = model.logits(torch.from_numpy(nxt)[:, None].to(gpu), False).float().cpu().numpy()[:, 0]
+
+
+def hf_model_from_state(cfg, sd, raw):
+    """The independent float64 model (tests/hf_formulation.py) over the dequantised weights of an
+    EET-named state dict; fused QKV columns are [Q | K | V] (modeling_llama.py:85)."""
+    import hf_formulation as HF
+    assert not cfg.alibi or cfg.heads & (cfg.heads - 1) == 0
+    slopes = HF.power_of_two_slopes(cfg.heads) if cfg.alibi else None
+    H = cfg.hidden
+
+    def deq(name):
+        q, s = raw[name]
+        return (q.numpy().astype(np.float64) * s.numpy().astype(np.float64)[None, :]).T      # [out, in]
+    layers = []
+    for i in range(cfg.num_layers):
+        pre = f"layer.{i}."
+        qkv = deq(pre + "self_attn.qkv_proj")
+        layers.append(HF.Layer(qkv[:H], qkv[H:2 * H], qkv[2 * H:], deq(pre + "self_attn.out_proj"),
+                               deq(pre + "ffn.intermediate_0"), deq(pre + "ffn.intermediate_1"), deq(pre + "ffn.output"),
+                               sd[pre + "self_attn.layernorm.weight"].numpy(), sd[pre + "ffn.layernorm.weight"].numpy(),
+                               cfg.heads, cfg.eps, slopes))
+    return HF.Model(sd["embed_tokens.weight"].numpy(), layers, sd["norm.weight"].numpy(),
+                    sd["lm_head.weight"].numpy(), cfg.eps)
+
+
+@pytest.mark.parametrize("alibi", [False, True])
+def test_decoder_matches_hf_formulation(gpu, alibi):
+    """The product against the independently written float64 model without a KV cache (teacher
+    forced: prefill 6 tokens, then 4 incremental calls), so a mistake shared by ops.py and the
+    oracle's composition would still show.  Error is relative to the RMS of the logits; the
+    product rounds to fp16 between ops, the independent model never does."""
+    cfg = tiny_cfg(alibi)
+    sd, raw = D.random_state_dict(cfg, seed=31)
+    model = D.Int8Decoder(cfg, sd, device="cuda:0")
+    hf = hf_model_from_state(cfg, sd, raw)
+    ids = torch.randint(0, cfg.vocab, (3, 10), generator=torch.Generator().manual_seed(5))
+    want = hf.logits(ids.numpy())
+    rms = np.sqrt((want * want).mean())
+    got = model.logits(ids[:, :6].to(gpu), True).float().cpu().numpy()[:, 0]
+    assert np.abs(got - want[:, 5]).max() / rms < 2e-2
+    for t in range(6, 10):
+        got = model.logits(ids[:, t:t + 1].to(gpu), False).float().cpu().numpy()[:, 0]
+        assert np.abs(got - want[:, t]).max() / rms < 2e-2, t
+
+
+@pytest.mark.parametrize("name", ["llama7b", "baichuan13b"])
+def test_full_width_layer(gpu, name):
+    """One decoder layer at the real width of benchmark configurations 4 and 5 (4096 / 32 heads /
+    11008 at batch 8; 5120 / 40 heads / 13696 with ALiBi at batch 32): a short prompt and two
+    incremental calls through the operator classes, against the oracle layer.
+    With K up to 13696 behind fp16 intermediates that the product and the oracle round at
+    different points, a handful of the ~10^5 outputs sit 2 fp16 steps apart at magnitude 4-8;
+    the per-element bound here is 2e-2 relative / 1e-2 absolute, backed by an RMS error bound
+    of 3e-3 over the tensor -- one to two fp16 steps of outputs of magnitude 1-4, which is what
+    two correct roundings of nearly equal fp32 values differ by (every linear of these shapes is held to 1e-2 / 1e-3 on its own in
+    test_gemm_gpu.py and test_config_shapes_gpu.py)."""
+    def close(got, want, what):
+        assert_close(got, want, 2e-2, 1e-2, what)
+        err = np.asarray(got, np.float32) - np.asarray(want, np.float32)
+        assert float(np.sqrt((err * err).mean())) < 3e-3, what
+    if name == "llama7b":
+        cfg = D.DecoderConfig(num_layers=1, hidden=4096, heads=32, d_ff=11008, vocab=64, alibi=False, max_batch=8,
+                              max_prompt=8, max_full_seq=12)
+    else:
+        cfg = D.DecoderConfig(num_layers=1, hidden=5120, heads=40, d_ff=13696, vocab=64, alibi=True, max_batch=32,
+                              max_prompt=8, max_full_seq=12)
+    eet_amd.ops.workspaces.clear()
+    sd, raw = D.random_state_dict(cfg, seed=41)
+    model = D.Int8Decoder(cfg, sd, device="cuda:0")
+    ref = oracle_decoder(cfg, sd, raw)
+    attn, ffn = model.layers[0]
+    oattn, offn = ref.layers[0]
+    g = torch.Generator().manual_seed(2)
+    B, S = cfg.max_batch, 5
+    e = torch.empty(0, dtype=torch.long)
+    x = torch.randn(B, S, cfg.hidden, generator=g).half()
+    print(f"full-width layer {name}: prefill B={B} S={S}", flush=True)
+    bias = D.alibi_mask(cfg.heads, S).to(gpu) if cfg.alibi else torch.empty(0)
+    y = attn.forward(x.to(gpu), e, e, True, True, True, bias)
+    want = oattn.forward(x.numpy(), None, True, O.alibi_mask(cfg.heads, S) if cfg.alibi else None)
+    close(y.cpu().numpy(), want, "attention prefill")
+    z = ffn.forward(y, True, True)
+    close(z.cpu().numpy(), offn.forward(y.cpu().numpy()), "ffn prefill")     # same input to both
+    for t in range(2):
+        step = S + t + 1
+        x1 = torch.randn(B, 1, cfg.hidden, generator=g).half()
+        print(f"full-width layer {name}: incremental call, step {step}", flush=True)
+        bias = D.alibi_mask(cfg.heads, step)[:, -1:, :].contiguous().to(gpu) if cfg.alibi else torch.empty(0)
+        y = attn.forward(x1.to(gpu), e, e, True, True, False, bias)
+        want = oattn.forward(x1.numpy(), None, False, O.alibi_bias(cfg.heads, step) if cfg.alibi else None)
+        close(y.cpu().numpy(), want, f"attention step {step}")
+        z = ffn.forward(y, True, True)
+        close(z.cpu().numpy(), offn.forward(y.cpu().numpy()), f"ffn step {step}")
+    del model
+    eet_amd.ops.workspaces.clear()
+    torch.cuda.empty_cache()

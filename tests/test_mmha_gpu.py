@@ -55,12 +55,12 @@ def test_against_oracle(gpu, B, H, dh, step, cap, use_pad, use_alibi):
 @pytest.mark.parametrize("threads", [256, 512, 1024])
 @pytest.mark.parametrize("ring", [2, 4, 8])
 @pytest.mark.parametrize("nsplit", [1, 3])
-def test_every_launch_shape(gpu, monkeypatch, threads, ring, nsplit):
+def test_every_launch_shape(gpu, tuning, threads, ring, nsplit):
     """Every workgroup width / ring depth / split count the kernel is instantiated for (selected with the
     tuning overrides), with padding, ALiBi, the fused rotary append and a ragged last pass of the ring."""
-    monkeypatch.setenv("EET_MMHA_THREADS", str(threads))
-    monkeypatch.setenv("EET_MMHA_UNROLL", str(ring))
-    monkeypatch.setenv("EET_MMHA_NSPLIT", str(nsplit))
+    tuning("EET_MMHA_THREADS", str(threads))
+    tuning("EET_MMHA_UNROLL", str(ring))
+    tuning("EET_MMHA_NSPLIT", str(nsplit))
     for (B, H, dh, step, use_pad, use_alibi) in [(2, 3, 128, 333, True, False), (2, 2, 64, 1207, False, True),
                                                  (1, 2, 32, 45, True, True), (3, 2, 128, 3, False, False),
                                                  (2, 2, 96, 290, True, True)]:

@@ -1,0 +1,242 @@
+"""Pins the oracle's composed layer and decoder (OracleAttention, OracleFFN, OracleDecoder) with
+checks that do not retype them:
+
+  * against tests/hf_formulation.py -- float64, Hugging Face formulation, no KV cache, the whole
+    sequence recomputed under a causal mask -- at every prompt row and every incremental step;
+  * negative controls: the same comparison with one plausible mistake planted in the independent
+    model (gate/up swapped, residual taken after the norm, rotary position off by one, K and V
+    column blocks swapped) must FAIL by a wide margin, so the comparison has the power to see them;
+  * closed forms: zero output-projection / down-projection weights give output == input bit for
+    bit; a one-token prompt gives x + Wo . v / (1 + 1e-6); the rotary position of incremental
+    step t is the prompt position t (an incremental call equals the last row of a longer prefill).
+"""
+import math
+
+import numpy as np
+import pytest
+
+import hf_formulation as HF
+from oracle import ops as O
+from oracle import quant as Q
+
+EPS = 1e-6
+
+
+def make_model(seed, layers=2, hidden=128, heads=4, d_ff=192, vocab=96, alibi=False, cap=16, batch=2):
+    """Random HF-style weights -> per-channel int8 (oracle quantiser) -> (independent float64 model
+    over the dequantised weights, oracle decoder over the int8 weights)."""
+    rng = np.random.default_rng(seed)
+    dh = hidden // heads
+
+    def linear(out_f, in_f):
+        w = (rng.standard_normal((out_f, in_f)) * 0.08).astype(np.float16)     # nn.Linear layout [out, in]
+        q, s = Q.quantize_ref128(np.ascontiguousarray(w.T))                    # EET layout [in, out]
+        deq = (q.astype(np.float64) * s.astype(np.float64)[None, :]).T         # back to [out, in]
+        return q, s, deq
+
+    slopes = HF.power_of_two_slopes(heads) if alibi else None
+    hf_layers, or_layers = [], []
+    for _ in range(layers):
+        (qq, qs, wq), (kq, ks, wk), (vq, vs, wv) = [linear(hidden, hidden) for _ in range(3)]
+        oq, os_, wo = linear(hidden, hidden)
+        gq, gs, wg = linear(d_ff, hidden)
+        uq, us, wu = linear(d_ff, hidden)
+        dq, ds, wd = linear(hidden, d_ff)
+        g1 = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float16)
+        g2 = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float16)
+        hf_layers.append(HF.Layer(wq, wk, wv, wo, wg, wu, wd, g1, g2, heads, EPS, slopes))
+        # fused QKV: columns [Q | K | V] (python/eet/transformers/modeling_llama.py:85)
+        qkv_q, qkv_s = np.concatenate([qq, kq, vq], 1), np.concatenate([qs, ks, vs])
+        or_layers.append((O.OracleAttention(batch, heads, dh, cap, qkv_q, qkv_s, oq, os_, g1, EPS, rope=not alibi),
+                          O.OracleFFN(gq, gs, uq, us, dq, ds, g2, EPS)))
+    embed = (rng.standard_normal((vocab, hidden)) * 0.5).astype(np.float16)
+    gf = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float16)
+    head = (rng.standard_normal((vocab, hidden)) * 0.08).astype(np.float16)
+    hf = HF.Model(embed, hf_layers, gf, head, EPS)
+    orc = O.OracleDecoder(embed, or_layers, gf, head, EPS, n_head=heads, alibi=alibi)
+    return hf, orc, rng
+
+
+def max_rel(got, want):
+    """Largest error relative to the RMS magnitude of the expected tensor."""
+    want = np.asarray(want, np.float64)
+    return float(np.abs(np.asarray(got, np.float64) - want).max() / math.sqrt((want * want).mean()))
+
+
+# the oracle rounds to fp16 between ops (as the reference's buffers do); the independent model never rounds
+TOL = 1.5e-2
+
+
+def run_teacher_forced(hf, orc, ids, S, pad=None):
+    """Oracle: prefill ids[:, :S], then one incremental call per remaining token.  Independent
+    model: one full forward over all T tokens.  Returns the per-step relative errors of the logits."""
+    B, T = ids.shape
+    want = hf.logits(ids, pad)
+    errs = [max_rel(orc.step(ids[:, :S], True, pad), want[:, S - 1])]
+    for t in range(S, T):
+        errs.append(max_rel(orc.step(ids[:, t:t + 1], False, pad), want[:, t]))
+    return errs
+
+
+@pytest.mark.parametrize("alibi", [False, True])
+def test_decoder_matches_hf_formulation(alibi):
+    hf, orc, rng = make_model(11, alibi=alibi)
+    ids = rng.integers(0, 96, (2, 9))
+    errs = run_teacher_forced(hf, orc, ids, S=5)
+    assert max(errs) < TOL, errs
+
+
+def test_decoder_matches_hf_formulation_left_padded():
+    """Left padding: padded key columns carry no weight; rotary positions stay the raw token
+    indices (csrc/core/self_add_bias.cu:393 uses the sequence index, padding included)."""
+    hf, orc, rng = make_model(12)
+    ids = rng.integers(0, 96, (2, 8))
+    pad = np.array([0, 2])
+    B, T = ids.shape
+    want = hf.logits(ids, pad)
+    got = orc.step(ids[:, :5], True, pad)
+    assert max_rel(got, want[:, 4]) < TOL
+    for t in range(5, T):
+        assert max_rel(orc.step(ids[:, t:t + 1], False, pad), want[:, t]) < TOL
+
+
+def test_every_prompt_row_of_a_layer():
+    """One layer, all rows of the prompt (the decoder test only sees the last row of each call)."""
+    hf, orc, rng = make_model(13, layers=1)
+    x = rng.standard_normal((2, 6, 128)).astype(np.float16)
+    attn, ffn = orc.layers[0]
+    got = ffn.forward(attn.forward(x, None, True))
+    want = hf.layers[0](x.astype(np.float64))
+    assert max_rel(got, want) < TOL
+    # and the attention sub-layer alone, so an error cannot hide behind the FFN
+    hf2, orc2, _ = make_model(13, layers=1)
+    assert max_rel(orc2.layers[0][0].forward(x, None, True), hf2.layers[0].attention(x.astype(np.float64), None)) < TOL
+
+
+class _Mistake:
+    """Plants one plausible mistake into the independent model."""
+
+    @staticmethod
+    def swap_gate_up(layer):
+        layer.w[4], layer.w[5] = layer.w[5], layer.w[4]
+
+    @staticmethod
+    def residual_after_norm(layer):
+        orig = layer.ffn
+
+        def ffn(h):
+            hn = HF.rms(h, layer.g_ffn, layer.eps)
+            return orig(h) - h + hn
+        layer.ffn = ffn
+
+    @staticmethod
+    def swap_k_v(layer):
+        layer.w[1], layer.w[2] = layer.w[2], layer.w[1]
+
+    @staticmethod
+    def rotary_off_by_one(layer):
+        real = HF.rope
+        orig = layer.attention
+
+        def attention(x, pad):
+            HF.rope = lambda t, pos: real(t, pos + (pos >= 5))     # incremental steps shifted by one
+            try:
+                return orig(x, pad)
+            finally:
+                HF.rope = real
+        layer.attention = attention
+
+    @staticmethod
+    def rotary_pairs_adjacent(layer):
+        """GPT-J style pairs (2i, 2i+1) instead of NeoX pairs (i, i + dh/2)."""
+        real = HF.rope
+        orig = layer.attention
+
+        def gptj(x, positions):
+            d = x.shape[-1]
+            inv_freq = 1.0 / (10000.0 ** (np.arange(0, d, 2, dtype=np.float64) / d))
+            ang = positions[:, None] * inv_freq[None, :]
+            c, s = np.cos(ang)[None, None], np.sin(ang)[None, None]
+            out = np.empty_like(x)
+            out[..., 0::2] = x[..., 0::2] * c - x[..., 1::2] * s
+            out[..., 1::2] = x[..., 1::2] * c + x[..., 0::2] * s
+            return out
+
+        def attention(x, pad):
+            HF.rope = gptj
+            try:
+                return orig(x, pad)
+            finally:
+                HF.rope = real
+        layer.attention = attention
+
+
+@pytest.mark.parametrize("mistake", ["swap_gate_up", "residual_after_norm", "swap_k_v", "rotary_off_by_one",
+                                     "rotary_pairs_adjacent"])
+def test_comparison_sees_planted_mistakes(mistake):
+    hf, orc, rng = make_model(11)
+    for layer in hf.layers:
+        getattr(_Mistake, mistake)(layer)
+    ids = rng.integers(0, 96, (2, 9))
+    errs = run_teacher_forced(hf, orc, ids, S=5)
+    assert max(errs) > 5 * TOL, (mistake, errs)
+
+
+def test_zero_projection_is_the_identity():
+    """With all-zero O-proj (down-proj) weights the sub-layer returns its input bit for bit:
+    the residual is the un-normalised input and is added exactly once."""
+    _, orc, rng = make_model(14, layers=1)
+    attn, ffn = orc.layers[0]
+    x = rng.standard_normal((2, 4, 128)).astype(np.float16)
+    attn.o_q = np.zeros_like(attn.o_q)
+    assert np.array_equal(attn.forward(x, None, True), x)
+    x1 = rng.standard_normal((2, 1, 128)).astype(np.float16)
+    assert np.array_equal(attn.forward(x1, None, False), x1)
+    ffn.d_q = np.zeros_like(ffn.d_q)
+    assert np.array_equal(ffn.forward(x), x)
+
+
+def test_one_token_prompt_closed_form():
+    """A prompt of one token attends only itself: ctx = v / (1 + 1e-6) and the sub-layer output is
+    x + Wo . ctx, whatever q and k are (so also whatever the rotary position is)."""
+    _, orc, rng = make_model(15, layers=1)
+    attn = orc.layers[0][0]
+    x = rng.standard_normal((2, 1, 128)).astype(np.float16)
+    got = attn.forward(x, None, True)
+    xn = HF.rms(x.astype(np.float64), attn.gamma.astype(np.float64), EPS)
+    wv = attn.qkv_q[:, 256:].astype(np.float64) * attn.qkv_s[256:].astype(np.float64)
+    wo = attn.o_q.astype(np.float64) * attn.o_s.astype(np.float64)
+    want = x.astype(np.float64) + ((xn @ wv) / (1 + 1e-6)) @ wo
+    assert max_rel(got, want) < 5e-3
+    assert attn.step == 1
+
+
+def test_incremental_call_equals_last_row_of_longer_prefill():
+    """Rotary position and cache row of incremental step t are those of prompt position t: feeding
+    tokens one by one gives what a prefill of the longer prompt gives in its last row."""
+    _, orc_a, rng = make_model(16, layers=1)
+    _, orc_b, _ = make_model(16, layers=1)
+    x = rng.standard_normal((2, 7, 128)).astype(np.float16)
+    a, b = orc_a.layers[0][0], orc_b.layers[0][0]
+    a.forward(x[:, :4], None, True)
+    for t in range(4, 7):
+        inc = a.forward(x[:, t:t + 1], None, False)
+        full = b.forward(x[:, :t + 1], None, True)
+        assert np.abs(inc[:, 0].astype(np.float32) - full[:, -1].astype(np.float32)).max() < 4e-3
+        assert a.step == b.step == t + 1
+        assert np.array_equal(a.k_cache[:, :, :t + 1], b.k_cache[:, :, :t + 1])
+
+
+def test_greedy_tokens_match_hf_formulation():
+    hf, orc, rng = make_model(17)
+    ids = rng.integers(0, 96, (2, 5))
+    toks = orc.greedy(ids, 4)
+    seq = ids
+    for t in range(4):
+        lg = hf.logits(seq)[:, -1]
+        top2 = np.sort(lg, -1)[:, -2:]
+        nxt = lg.argmax(-1)
+        for b in range(2):
+            if top2[b, 1] - top2[b, 0] > 0.05:        # margin above the fp16 noise of the oracle
+                assert toks[b, t] == nxt[b]
+        seq = np.concatenate([seq, toks[:, t:t + 1]], 1)     # follow the oracle's tokens

@@ -5,6 +5,8 @@ import ctypes
 import json
 import os
 
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -133,6 +135,35 @@ def test_invariants():
     assert qq[:, 0].tolist() == [127, 3, -3, 1, -1, 2, -2, 0]
 
 
+def test_sym127_scalar_brute_force():
+    """quantize_sym127 against a scalar loop in C-float arithmetic (numpy float32 scalars):
+    scale = absmax / 127, q = round-half-away(w / scale) in [-127, 127], zero column -> 0."""
+    rng = np.random.default_rng(4)
+    w = (rng.standard_normal((24, 6)) * 0.02).astype(np.float32)
+    w[:, 1] = 0
+    w[3, 2], w[4, 2], w[5, 2] = 127.0, 2.5, -0.5           # scale exactly 1: ties visible
+    w[:3, 2] = [1.5, -1.5, 126.5]
+    q, s = Q.quantize_sym127(w)
+    for n in range(w.shape[1]):
+        amax = np.float32(0)
+        for k in range(w.shape[0]):
+            amax = max(amax, np.float32(abs(w[k, n])))
+        sc = np.float32(amax / np.float32(127.0))
+        assert s[n] == sc
+        for k in range(w.shape[0]):
+            if sc == 0:
+                want = 0
+            else:
+                r = float(np.float32(w[k, n] / sc))
+                want = int(math.copysign(math.floor(abs(r) + 0.5), r))     # exact in float64
+                want = max(-127, min(127, want))
+            assert q[k, n] == want, (k, n)
+    assert q[3, 2] == 127 and q[4, 2] == 3 and q[5, 2] == -1 and q[0, 2] == 2 and q[1, 2] == -2 and q[2, 2] == 127
+    # the extreme element of a non-zero column is exactly +-127
+    k = np.abs(w).argmax(0)
+    assert (np.abs(q[k, np.arange(6)].astype(int))[[0, 2, 3, 4, 5]] == 127).all()
+
+
 def test_sym127_generator():
     rng = np.random.default_rng(3)
     w = (rng.standard_normal((128, 32)) * 0.02).astype(np.float16)
@@ -234,9 +265,13 @@ def test_torch_packer_and_quantiser_match_the_library():
     assert torch.equal(eet_amd.pack_weights_torch(q), eet_amd.pack_weights(q))
     w = torch.from_numpy((rng.standard_normal((512, 64)) * 0.02).astype(np.float16))
     w[:, 3] = 0
+    # a column whose scale is exactly 1 (ref128) with exact ties and the value just below one half,
+    # where floor(|x| + 0.5) would round up and C round() does not
+    w32 = w.float()
+    w32[:, 5] = 0
+    w32[:8, 5] = torch.tensor([128.0, 2.5, -2.5, 0.5, -0.5, 0.49999997, -0.49999997, 127.5])
     for mode in ("ref128", "sym127"):
-        u, p, s = eet_amd.quant_weights(w, torch.int8, True, mode=mode)
-        ut, st = eet_amd.quant_weights_torch(w, mode)
-        # |x| + 0.5 can round up in fp32 where C round() does not; such ties-by-rounding are
-        # vanishingly rare for Gaussian data, and the torch path is a data generator, not the packer
-        assert (ut != u).sum() <= 1 and torch.equal(st, s)
+        for mat in (w, w32):
+            u, p, s = eet_amd.quant_weights(mat, torch.int8, True, mode=mode)
+            ut, st = eet_amd.quant_weights_torch(mat, mode)
+            assert torch.equal(ut, u) and torch.equal(st, s)

@@ -485,3 +485,66 @@ extern "C" int eet_mmha_decode(const void *q, const void *k, const void *v, long
     return run_mmha(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, dh, step, T_cap, rope_cos_sin,
                     workspace, plan, static_cast<hipStream_t>(stream));
 }
+
+// ---------------------------------------------------------------------------
+// The same call for callers that cannot allocate: the split partials live in a
+// file-scope device array instead of a caller-supplied workspace.
+// ---------------------------------------------------------------------------
+namespace {
+
+// Largest split launch the static entry point takes: B*H*nsplit <= 512 partial
+// records of (max, sum, acc[dh <= 128]) floats.  The table splits only when
+// B*H < 256 and never into more than ceil(256 / (B*H)) parts, so every shape it
+// chooses by itself fits (B*H*nsplit < 256 + B*H).
+constexpr size_t kScratchRecords = 512;
+constexpr size_t kScratchFloats = kScratchRecords * (128 + 2);
+
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+// Device address of `scratch` per GPU (each device holds its own copy of the
+// array at its own address); looked up once per device, with that device current.
+constexpr int kMaxDevices = 64;
+float *g_scratch_ptr[kMaxDevices];
+
+int scratch_for_current_device(float **out)
+{
+    int dev = -1;
+    EET_HIP_CHECK(hipGetDevice(&dev));
+    EET_REQUIRE(dev >= 0 && dev < kMaxDevices, EET_ERR_HIP, "eet_mmha_decode_static: device ordinal %d out of range", dev);
+    float *p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (p == nullptr) {
+        void *addr = nullptr;
+        EET_HIP_CHECK(hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)));
+        EET_REQUIRE(addr != nullptr, EET_ERR_HIP, "eet_mmha_decode_static: no device address for the scratch array");
+        p = static_cast<float *>(addr);
+        __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);  // racing threads store the same address
+    }
+    *out = p;
+    return EET_OK;
+}
+
+}  // namespace
+
+extern "C" size_t eet_mmha_decode_static_capacity(void) { return kScratchFloats * sizeof(float); }
+
+extern "C" int eet_mmha_decode_static(const void *q, const void *k, const void *v, long qkv_stride, void *k_cache,
+                                      void *v_cache, void *ctx, const void *alibi, const int64_t *pad, int B, int H,
+                                      int dh, int step, int T_cap, const float *rope_cos_sin, void *stream)
+{
+    Plan plan;
+    if (int rc = check_mmha_args("eet_mmha_decode_static", q, k, v, qkv_stride, k_cache, v_cache, ctx, B, H, dh, step,
+                                 T_cap, rope_cos_sin, &plan))
+        return rc;
+    const size_t need = plan.nsplit > 1 ? (size_t)B * H * plan.nsplit * (dh + 2) * sizeof(float) : 0;
+    EET_REQUIRE(need <= kScratchFloats * sizeof(float), EET_ERR_WORKSPACE,
+                "eet_mmha_decode_static: B*H*nsplit = %d*%d*%d partial records (%zu bytes) exceed the static scratch of "
+                "%zu bytes; use eet_mmha_decode with a workspace",
+                B, H, plan.nsplit, need, kScratchFloats * sizeof(float));
+    float *partials = nullptr;
+    if (int rc = scratch_for_current_device(&partials))
+        return rc;
+    // Every partial record a launch reads was written by the same launch's first
+    // kernel, so nothing has to be cleared between calls.
+    return run_mmha(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, dh, step, T_cap, rope_cos_sin,
+                    partials, plan, static_cast<hipStream_t>(stream));
+}

@@ -174,6 +174,23 @@ int eet_mmha_decode(const void *q, const void *k, const void *v, long qkv_stride
                     const float *rope_cos_sin, void *workspace, size_t workspace_bytes,
                     void *stream);
 
+/* eet_mmha_decode for callers that cannot allocate device memory or carry a
+ * workspace around: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  It has no counterpart in the reference.  Same
+ * arguments and results as eet_mmha_decode, without the workspace: the partial
+ * results of a split launch (B*H < 256) live in a static device array of
+ * eet_mmha_decode_static_capacity() bytes (260 KiB) that every GPU the library
+ * runs on holds until the process ends.  Calls no hipMalloc / hipFree.  A call
+ * whose B*H*nsplit*(dh+2)*4 bytes exceed the capacity (only reachable through a
+ * tuning override) fails with EET_ERR_WORKSPACE.  All calls on one GPU share the
+ * array: calls that overlap in time on different streams of one GPU race;
+ * nothing needs clearing between calls. */
+size_t eet_mmha_decode_static_capacity(void);
+int eet_mmha_decode_static(const void *q, const void *k, const void *v, long qkv_stride,
+                           void *k_cache, void *v_cache, void *ctx, const void *alibi,
+                           const int64_t *pad, int B, int H, int dh, int step, int T_cap,
+                           const float *rope_cos_sin, void *stream);
+
 /* table[t][0 .. dh/2) = cos(t / 10000^(2i/dh)), table[t][dh/2 .. dh) = sin(...),
  * t in [0, T): the rotary coefficients of csrc/core/common.cuh:176-180 in fp32. */
 int eet_rope_table(float *table, int T, int dh, void *stream);

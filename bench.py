@@ -3,9 +3,10 @@
 plus LLaMA-7B-shaped int8 decode tokens/s, on one MI355X.
 
 A "step" is one pass of the fused dequant-GEMM over every int8 linear of a
-32-layer LLaMA-7B-shaped decoder (160 launches over 6.48 GB of distinct packed
-weights, so nothing is served from the 256 MB Infinity Cache) at M = 8 rows of
-fp16 activations.  `value` is algorithmic bytes per step / time per step.
+32-layer LLaMA-7B-shaped decoder, launched as the decoder ops launch them (128
+launches over 6.48 GB of distinct packed weights, so nothing is served from the
+256 MB Infinity Cache) at M = 8 rows of fp16 activations.  `value` is
+algorithmic bytes per step / time per step.
 
 Prints ONE JSON line.  Synthetic, seeded data; weights live in HBM before the
 timed region starts.
@@ -36,11 +37,6 @@ def linear_shapes(hidden, d_ff):
 EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 
 
-def launch_shapes(hidden, d_ff):
-    return [("qkv", hidden, 3 * hidden, EPI_NONE), ("o+residual", hidden, hidden, EPI_RESIDUAL),
-            ("gate|up+swiglu", hidden, 2 * d_ff, EPI_SWIGLU), ("down+residual", d_ff, hidden, EPI_RESIDUAL)]
-
-
 def linear_bytes(M, K, N, epi=EPI_NONE):
     """Algorithmic bytes of one int8 linear: each operand once (weights, scales, activations,
     output; plus the residual rows read by that epilogue; the SwiGLU output is M x N/2)."""
@@ -65,19 +61,26 @@ def make_weights(torch, eet, dev, layers, hidden, d_ff, seed):
     return out
 
 
+RMS_LAUNCHES = ("rmsnorm+qkv", "rmsnorm+gate|up+swiglu")     # the launches that carry the RMSnorm prologue
+
+
 def fused_launch_weights(eet_ops, weights):
-    """Per layer, the operands of the four launches of launch_shapes()."""
+    """Per layer, the operands of the four launches the decoder ops make (eet_amd/csrc/decode_ops.cc):
+    RMSnorm + QKV, O + residual, RMSnorm + gate|up + SwiGLU, down + residual."""
     out = []
     for layer in weights:
         w01, s01 = eet_ops.interleave_gate_up(layer["gate"][0], layer["gate"][1], layer["up"][0], layer["up"][1])
-        out.append({"qkv": layer["qkv"] + (EPI_NONE,), "o+residual": layer["o"] + (EPI_RESIDUAL,),
-                    "gate|up+swiglu": (w01, s01, EPI_SWIGLU), "down+residual": layer["down"] + (EPI_RESIDUAL,)})
+        out.append({"rmsnorm+qkv": layer["qkv"] + (EPI_NONE,), "o+residual": layer["o"] + (EPI_RESIDUAL,),
+                    "rmsnorm+gate|up+swiglu": (w01, s01, EPI_SWIGLU), "down+residual": layer["down"] + (EPI_RESIDUAL,)})
     return out
 
 
-def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup):
+def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup, probe=False, probe_grid_scale=1):
     """Returns seconds per step (one pass over all linears), measured with
-    events on the stream the kernels are launched on."""
+    events on the stream the kernels are launched on.  Launches named in
+    RMS_LAUNCHES carry the RMSnorm prologue, as in the decoder.  probe=True
+    replaces every GEMM by the read-only streaming probe over the same weight
+    buffer with the same grid (the machine's ceiling for this launch chain)."""
     st = torch.cuda.current_stream()
     calls = []
     for layer in weights:
@@ -85,15 +88,27 @@ def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup):
             K, N = w.shape
             n_out = N // 2 if epi == EPI_SWIGLU else N
             res = outs["residual"].data_ptr() if epi == EPI_RESIDUAL else None
-            calls.append((acts[K].data_ptr(), w.data_ptr(), s.data_ptr(), outs[n_out].data_ptr(), M, N, K, epi, res))
+            gam = outs["gamma"].data_ptr() if name in RMS_LAUNCHES else None
+            calls.append((acts[K].data_ptr(), w.data_ptr(), s.data_ptr(), outs[n_out].data_ptr(), M, N, K, epi, res, gam))
     f = lib.eet_gemm_w8a16_fused
     sp = st.cuda_stream
 
-    def one_pass():
-        for (a, w, s, c, m, n, k, epi, res) in calls:
-            rc = f(a, w, s, c, m, n, k, epi, res, None, 0.0, None, 0, sp)
-            if rc:
-                raise RuntimeError(lib.eet_last_error().decode())
+    if probe:
+        sink = outs["probe_sink"]
+        g = lib.eet_hbm_stream_probe
+
+        def one_pass():
+            for (a, w, s, c, m, n, k, epi, res, gam) in calls:
+                # the grid the GEMM uses for this shape: 256 workgroups, 688 for the merged gate|up matrix
+                rc = g(w, k * n, (688 if epi == EPI_SWIGLU else 256) * probe_grid_scale, sink.data_ptr(), sink.numel(), sp)
+                if rc:
+                    raise RuntimeError(lib.eet_last_error().decode())
+    else:
+        def one_pass():
+            for (a, w, s, c, m, n, k, epi, res, gam) in calls:
+                rc = f(a, w, s, c, m, n, k, epi, res, gam, 1e-6, None, 0, sp)
+                if rc:
+                    raise RuntimeError(lib.eet_last_error().decode())
     for _ in range(warmup):
         one_pass()
     torch.cuda.synchronize()
@@ -108,12 +123,37 @@ def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup):
     return e0.elapsed_time(e1) * 1e-3 / steps, wall, len(calls)
 
 
-def cpu_baseline(torch, M, hidden, d_ff, seed, budget_s=12.0):
+def cpu_info():
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for line in fh:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return model
+
+
+def cpu_threads():
+    """Threads the CPU legs run on: every core the process may use (the GPU boxes give a job
+    16 cores whatever os.cpu_count() says)."""
+    try:
+        allowed = len(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = os.cpu_count() or 1
+    return max(1, min(allowed, int(os.environ.get("OMP_NUM_THREADS", allowed))))
+
+
+def cpu_baseline(torch, M, hidden, d_ff, seed, budget_s=10.0):
     """The reference CPU path, timed on the host cores: torch dequantise
     (int8 * scale -> fp32) + fp32 matmul -> fp16, for one layer's five linears
-    (the same shapes as the GPU workload; a bounded sample of it)."""
+    (the same shapes as the GPU workload; a bounded sample of it).  Also timed:
+    the matmul alone with the dequantised fp32 weights kept (the second number
+    the reference path could be quoted on)."""
     from oracle import cpu_path
-    threads = min(os.cpu_count() or 1, 16)
+    threads = cpu_threads()
     torch.set_num_threads(threads)
     g = torch.Generator().manual_seed(seed)
     layer = []
@@ -132,10 +172,65 @@ def cpu_baseline(torch, M, hidden, d_ff, seed, budget_s=12.0):
         if el > budget_s or reps >= 20:
             break
     per_layer = el / reps
+    # matmul only: weights dequantised once, outside the timed region
+    cached = [(x.float(), q.float() * s.float()[None, :]) for x, q, s in layer]
+    for x32, wd in cached:
+        (x32 @ wd).half()
+    reps2, t0 = 0, time.perf_counter()
+    while True:
+        for x32, wd in cached:
+            (x32 @ wd).half()
+        reps2 += 1
+        el2 = time.perf_counter() - t0
+        if el2 > budget_s / 2 or reps2 >= 20:
+            break
+    per_layer_mm = el2 / reps2
     return {"value": round(nbytes / per_layer / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"one LLaMA-7B layer (5 int8 linears, M={M}, {nbytes / 1e6:.1f} MB algorithmic), "
                       f"{reps} reps, torch {torch.__version__} dequant+matmul fp32, "
-                      f"{per_layer * 1e3:.1f} ms per layer"}
+                      f"{per_layer * 1e3:.1f} ms per layer",
+            "matmul_only_value": round(nbytes / per_layer_mm / 1e9, 3),
+            "matmul_only_sample": f"same layer, fp32 weights dequantised beforehand, {reps2} reps, "
+                                  f"{per_layer_mm * 1e3:.1f} ms per layer",
+            "os_cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads(), "cpu_model": cpu_info()}
+
+
+def cpu_decode_baseline(torch, model, batch, step, layers_timed=2, steps_timed=2, seed=11):
+    """One token step of the CPU oracle decoder (numpy fp32: dequantise + matmul, attention over
+    the fp16 KV cache) at the decoder's real width, on `layers_timed` layers with KV caches
+    filled with N(0,1) rows up to `step`, extrapolated to the full depth (labelled as such)."""
+    import numpy as np
+
+    from oracle import ops as O
+    rng = np.random.default_rng(seed)
+    H, heads, F = model["hidden"], model["heads"], model["d_ff"]
+    dh = H // heads
+
+    def lin(K, N):
+        return rng.integers(-128, 128, (K, N), dtype=np.int8), (rng.random(N) * 1e-3 + 1e-4).astype(np.float16)
+    layers = []
+    for _ in range(layers_timed):
+        gam = np.ones(H, np.float16)
+        attn = O.OracleAttention(batch, heads, dh, step + steps_timed + 2, *lin(H, 3 * H), *lin(H, H), gam, 1e-6,
+                                 rope=not model["alibi"])
+        attn.k_cache[:, :, :step] = rng.standard_normal((batch, heads, step, dh), dtype=np.float32).astype(np.float16)
+        attn.v_cache[:, :, :step] = rng.standard_normal((batch, heads, step, dh), dtype=np.float32).astype(np.float16)
+        attn.step = step
+        layers.append((attn, O.OracleFFN(*lin(H, F), *lin(H, F), *lin(F, H), gam, 1e-6)))
+    x = rng.standard_normal((batch, 1, H), dtype=np.float32).astype(np.float16)
+    t0 = time.perf_counter()
+    for t in range(steps_timed):
+        y = x
+        for attn, ffn in layers:
+            bias = O.alibi_bias(heads, attn.step + 1) if model["alibi"] else None
+            y = ffn.forward(attn.forward(y, None, False, bias))
+    per_layer = (time.perf_counter() - t0) / (steps_timed * layers_timed)
+    step_s = per_layer * model["layers"]
+    return {"tokens_per_s_extrapolated": round(batch / step_s, 3), "s_per_token_step_extrapolated": round(step_s, 3),
+            "measured": f"{layers_timed} layers x {steps_timed} token steps of the numpy fp32 oracle decoder at hidden {H}, "
+                        f"batch {batch}, cache length {step}: {per_layer * 1e3:.0f} ms per layer; multiplied by "
+                        f"{model['layers']} layers (embedding, final norm and lm_head not included)",
+            "cores": cpu_threads(), "kind": "port"}
 
 
 def device_packer_bench(torch, eet, lib, dev, iters=3):
@@ -187,7 +282,7 @@ def packer_bench(torch, eet):
     eet.quant_weights(w, torch.int8, False)
     t_ours = time.perf_counter() - t0
     out = {"shape": f"K={K} N={N} fp16", "quantise_and_pack_s": round(t_ours, 3),
-           "Mweights_per_s": round(K * N / t_ours / 1e6, 1), "threads": min(os.cpu_count() or 1, 16)}
+           "Mweights_per_s": round(K * N / t_ours / 1e6, 1), "threads": cpu_threads()}
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "oracle", "liboracle.so")
     if os.path.exists(path):
         ref = ctypes.CDLL(path)
@@ -211,7 +306,7 @@ def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed, model=LLAMA
     from eet_amd import decoder as D
     cfg = D.DecoderConfig(num_layers=len(weights), hidden=model["hidden"], heads=model["heads"], d_ff=model["d_ff"],
                           vocab=model["vocab"], alibi=model["alibi"], max_batch=batch, max_prompt=prompt,
-                          max_full_seq=prompt + gen + 1)
+                          max_full_seq=prompt + gen + 10)
     g = torch.Generator(device=dev).manual_seed(seed)
     H = cfg.hidden
     sd = {}
@@ -249,8 +344,36 @@ def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed, model=LLAMA
             nxt = torch.argmax(logits[:, -1, :], dim=-1)
         torch.cuda.synchronize()
         t_dec = time.perf_counter() - t0
+        # per-kernel breakdown from further steps of the same run: each launch issued on its own
+        # and bracketed by events (the timed loop above used the one-call-per-op path)
+        from eet_amd import ops as _ops
+        timer = _ops.LaunchTimer()
+        _ops.launch_timer = timer
+        bd_steps = min(8, max(0, cfg.max_full_seq - (prompt + gen) - 1))
+        try:
+            for _ in range(bd_steps):
+                logits = model.logits(nxt[:, None], False)
+                nxt = timer.run("argmax (torch)", batch * cfg.vocab * 2, lambda: torch.argmax(logits[:, -1, :], dim=-1))
+        finally:
+            _ops.launch_timer = None
+        raw = timer.summary() if bd_steps else {}
     steps = gen - 1
     ms = t_dec / steps * 1e3
+    # A bracket (event, launch, event) costs more than the launch does back to back -- the two event
+    # records are packets of their own -- so the bracketed times are scaled to sum to the step time
+    # measured without them; both are given.
+    breakdown = {}
+    tot = sum(r["us_total"] for r in raw.values()) / max(bd_steps, 1)
+    for name, r in raw.items():
+        us_raw = r["us_total"] / r["calls"]
+        us = us_raw * (ms * 1e3 / tot)
+        gbs = (r["bytes_total"] / r["calls"]) / us / 1e3
+        breakdown[name] = {"calls_per_step": r["calls"] // bd_steps, "us_per_call": round(us, 2),
+                           "us_per_call_bracketed": round(us_raw, 2),
+                           "us_per_step": round(us * (r["calls"] // bd_steps), 1),
+                           "share_of_step": round(r["us_total"] / bd_steps / tot, 4),
+                           "bytes_per_call": r["bytes_total"] // r["calls"], "GB/s": round(gbs, 1),
+                           "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
     # algorithmic HBM bytes of one token step: int8 weights + scales, KV cache read at mid length, fp16 lm_head
     wbytes = sum(w.numel() + 2 * s.numel() for layer in weights for (w, s) in layer.values())
     kv = len(weights) * 2 * (prompt + gen // 2) * batch * H * 2
@@ -259,6 +382,10 @@ def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed, model=LLAMA
             "prompt": prompt, "generated": gen, "layers": len(weights), "prefill_s": round(t_prefill, 3), "prefill_warm_s": round(t_prefill_warm, 3),
             "step_hbm_bytes": step_bytes,
             "step_roofline_frac": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "breakdown": breakdown,
+            "breakdown_note": f"{bd_steps} further token steps with every launch issued on its own between two events; "
+                              "us_per_call is the bracketed time scaled so that the kernels of a step sum to "
+                              "ms_per_token_step (the brackets themselves cost time); bytes are algorithmic",
             "note": "greedy decode, random-init weights, random token ids; lm_head and embedding are fp16 torch ops"}
 
 
@@ -294,6 +421,41 @@ def prefill_gemm_bench(torch, eet, lib, dev, iters=10):
         tf = 2.0 * M * N * K / t / 1e12
         out[f"{name} M={M} K={K} N={N}"] = {"us": round(t * 1e6, 1), "TFLOP/s": round(tf, 1),
                                             "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4)}
+    return out
+
+
+def prefill_attention_bench(torch, lib, dev, iters=5):
+    """Causal prefill attention (flash-style MFMA kernel) at the prompt shapes of configurations 4 and 5:
+    TFLOP/s over the causal half of the work, 4 * B * H * (S^2 / 2) * dh."""
+    out = {}
+    st = torch.cuda.current_stream()
+    for name, B, H, S, alibi in (("llama7b B=8 H=32 S=1024", 8, 32, 1024, False),
+                                 ("baichuan13b B=8 H=40 S=2048 alibi", 8, 40, 2048, True),
+                                 ("baichuan13b B=8 H=40 S=2048 no bias", 8, 40, 2048, False)):
+        dh = 128
+        g = torch.Generator(device=dev).manual_seed(S)
+        q, kc, vc = [torch.randn(B, H, S, dh, generator=g, device=dev).half() for _ in range(3)]
+        ctx = torch.empty(B, S, H * dh, dtype=torch.float16, device=dev)
+        bias = (torch.rand(H, S, generator=g, device=dev) * 8).half() if alibi else None
+
+        def call():
+            rc = lib.eet_prefill_attention(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), ctx.data_ptr(),
+                                           bias.data_ptr() if alibi else None, None, B, H, S, dh, S, st.cuda_stream)
+            if rc:
+                raise RuntimeError(lib.eet_last_error().decode())
+        for _ in range(2):
+            call()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(st)
+        for _ in range(iters):
+            call()
+        e1.record(st)
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e-3 / iters
+        tf = 4.0 * B * H * (S * S / 2) * dh / t / 1e12
+        out[name] = {"us": round(t * 1e6, 1), "TFLOP/s_causal": round(tf, 1),
+                     "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4)}
     return out
 
 
@@ -341,6 +503,22 @@ def attention_bench(torch, lib, dev, iters=20):
     return out
 
 
+def recorded_traffic(M, layers):
+    """HBM-side bytes per launch of the headline pass as recorded in profiles/ (a line
+    'traffic_bytes_per_launch M=<M> layers=<n>: <bytes>' in the pmc summary), or None."""
+    import glob
+    import re
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*pmc*"))):
+        try:
+            text = open(path).read()
+        except OSError:
+            continue
+        m = re.search(rf"traffic_bytes_per_launch M={M} layers={layers}: (\d+)", text)
+        if m:
+            return int(m.group(1))
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -353,9 +531,12 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the M = 1..32 sweep")
-    ap.add_argument("--baichuan", action="store_true",
-                    help="also run benchmark configuration 5: Baichuan-13B-shaped decoder (40 layers, ALiBi), batch 32, "
+    ap.add_argument("--no-baichuan", action="store_true",
+                    help="skip benchmark configuration 5: Baichuan-13B-shaped decoder (40 layers, ALiBi), batch 32, "
                          "prompt 2048, 256 greedy tokens (needs ~85 GB of HBM and about a minute)")
+    ap.add_argument("--only", default="",
+                    help="comma-separated extra legs to run instead of all of them (for profiling one kernel): "
+                         "prefill_gemm, prefill_attention, decode_attention, packer_device")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 1 GiB device-to-device copies (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -381,6 +562,8 @@ def main():
     acts = {K: torch.randn(32, K, generator=g, device=dev).half() for K in (hidden, d_ff)}
     outs = {N: torch.empty(32, N, dtype=torch.float16, device=dev) for N in (3 * hidden, hidden, d_ff)}
     outs["residual"] = torch.randn(32, hidden, generator=g, device=dev).half()
+    outs["gamma"] = (1 + 0.1 * torch.randn(hidden, generator=g, device=dev)).half()
+    outs["probe_sink"] = torch.empty(4 * 1024 * 1024, dtype=torch.uint8, device=dev)
     from eet_amd import ops as eet_ops
     fused = fused_launch_weights(eet_ops, weights)
 
@@ -392,6 +575,12 @@ def main():
     step_bytes = pass_bytes(fused, M)
     gbs = step_bytes / sec / 1e9
     per_launch_us = sec / launches * 1e6
+    # the same chain of launches as pure reads of the same weight buffers: what the machine allows
+    # (with the GEMM's own grids, and with two and four times as many workgroups: the best of the three counts)
+    probe_sec = min(time_gemm_pass(torch, L, fused, acts, outs, M, max(3, args.steps // 2), 1, probe=True,
+                                   probe_grid_scale=sc)[0] for sc in (1, 2, 4))
+    weight_bytes = sum(w.numel() for layer in fused for (w, _, _) in layer.values())
+    ceiling_gbs = weight_bytes / probe_sec / 1e9
     result = {
         "metric": "int8 W-only GEMM HBM GB/s (% peak) at M=1..16; LLaMA-7B int8 decode tokens/s, 1 GPU",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -399,17 +588,24 @@ def main():
         "dtype": "fp16 activations x int8 weights, fp32 accumulate", "data": "synthetic",
         "config": {"workload": f"LLaMA-7B-shaped decode linears, int8 per-channel weights: {args.layers} layers x "
                                f"(QKV 4096x12288, O 4096x4096, gate/up 4096x11008, down 11008x4096) at M={M}, "
-                               "launched as the decoder ops launch them: gate and up in one launch with the "
-                               "SwiGLU epilogue, O and down with the residual-add epilogue",
+                               "launched as the decoder ops launch them: RMSnorm prologue on QKV, gate and up in "
+                               "one launch with the RMSnorm prologue and the SwiGLU epilogue, O and down with the "
+                               "residual-add epilogue",
                    "launches_per_step": launches, "bytes_per_step": step_bytes,
                    "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "kernel": "w8a16_small_m_kernel", "achieved": round(gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "avg_launch_us": round(per_launch_us, 3),
                      "algorithmic_bytes_per_launch": round(step_bytes / launches),
-                     # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE (x2.000, calibrated on a
-                     # 1 GiB copy) + WRITE_SIZE (x1.000) at the default workload (measured once, not per run)
-                     "traffic": 51.73e6 if (M == 8 and args.layers == 32) else None},
+                     # HBM-side bytes per launch, from the committed rocprofv3 --pmc summary of this workload
+                     # (FETCH_SIZE and WRITE_SIZE scaled by a copy kernel of known size); null if none matches
+                     "traffic": recorded_traffic(M, args.layers),
+                     "stream_ceiling": {"GB/s": round(ceiling_gbs, 1), "frac_of_peak": round(ceiling_gbs / HBM_PEAK_GBS, 4),
+                                        "ms_per_step": round(probe_sec * 1e3, 4),
+                                        "what": "the same 128 launches per step as read-only streams of the same weight "
+                                                "buffers (eet_hbm_stream_probe, same grids): the rate this machine "
+                                                "allows a chain of dependent launches of these sizes"},
+                     "frac_of_stream_ceiling": round(step_bytes / sec / (weight_bytes / probe_sec), 4)},
         "host_wall_ms_per_step": round(wall * 1e3, 4),
     }
 
@@ -429,7 +625,7 @@ def main():
             sweep[f"M={m}"] = {"GB/s": round(b / s / 1e9, 1), "pct_peak": round(100 * b / s / 1e9 / HBM_PEAK_GBS, 2)}
         per_shape = {}
         plain = [{k: v + (EPI_NONE,) for k, v in layer.items()} for layer in weights]
-        for src, names in ((fused, [n for n, _, _, _ in launch_shapes(hidden, d_ff)]), (plain, ["gate", "up"])):
+        for src, names in ((fused, list(fused[0].keys())), (plain, ["gate", "up"])):
             for name in names:
                 sub = [{name: layer[name]} for layer in src]
                 s, _, n = time_gemm_pass(torch, L, sub, acts, outs, M, max(3, args.steps // 4), 1)
@@ -441,19 +637,28 @@ def main():
         result["gemm_by_m"] = sweep
         result[f"gemm_by_shape_M{M}"] = per_shape
 
-    if not args.no_sweep:
+    only = [x for x in args.only.split(",") if x]
+    if (not args.no_sweep and not only) or "prefill_gemm" in only:
         result["prefill_gemm_config3"] = prefill_gemm_bench(torch, eet, L, dev)
+    if (not args.no_sweep and not only) or "prefill_attention" in only:
+        result["prefill_attention"] = prefill_attention_bench(torch, L, dev)
+    if (not args.no_sweep and not only) or "decode_attention" in only:
         result["decode_attention"] = attention_bench(torch, L, dev)
+    if (not args.no_sweep and not only) or "packer_device" in only:
         result["packer_device"] = device_packer_bench(torch, eet, L, dev)
 
     if args.gen > 0:
         result["decode"] = decode_bench(torch, eet, weights, dev, args.batch, args.prompt, args.gen, seed=7)
 
-    if args.baichuan:
+    if not args.no_cpu and args.gen > 0:
+        result["decode"]["cpu_baseline"] = cpu_decode_baseline(torch, LLAMA, args.batch, args.prompt + args.gen // 2)
+
+    if not args.no_baichuan:
         del weights, fused
         torch.cuda.empty_cache()
         from eet_amd import ops as _ops
         _ops.workspaces.clear()
+        _ops.spare_kv.clear()
         bw = make_weights(torch, eet, dev, BAICHUAN13B["layers"], BAICHUAN13B["hidden"], BAICHUAN13B["d_ff"], seed=4321)
         result["decode_baichuan13b"] = decode_bench(torch, eet, bw, dev, 32, 2048, 256, seed=9, model=BAICHUAN13B)
         del bw

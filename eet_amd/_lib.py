@@ -40,6 +40,7 @@ SIGNATURES = {
     "eet_swiglu": (_i, [_vp, _vp, _i, _i, _vp]),
     "eet_residual_add": (_i, [_vp, _vp, _i, _i, _vp]),
     "eet_kv_cache_reorder": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "eet_hbm_stream_probe": (_i, [_vp, _sz, _i, _vp, _sz, _vp]),
     "eet_prefill_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
 }
 

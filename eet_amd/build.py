@@ -12,7 +12,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libeet_hip.so")
 
-SOURCES = ["packer.cc", "tuning.cc", "decode_ops.cc", "packer_device.hip", "gemm_w8a16.hip", "gemm_w8a16_large.hip", "mmha_decode.hip", "prefill_attention.hip", "glue.hip"]
+SOURCES = ["packer.cc", "tuning.cc", "decode_ops.cc", "packer_device.hip", "gemm_w8a16.hip", "gemm_w8a16_large.hip", "mmha_decode.hip", "prefill_attention.hip", "glue.hip", "probe.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

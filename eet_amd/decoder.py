@@ -157,7 +157,8 @@ class Int8Decoder:
             pad = self.pre_padding_len
         else:
             pad = torch.sum(1 - attention_mask, 1, True).to(input_ids.device).long()
-        x = torch.nn.functional.embedding(input_ids, self.embed)
+        x = ops._timed("embedding (torch)", 2 * B * S * cfg.hidden * 2,
+                       lambda: torch.nn.functional.embedding(input_ids, self.embed))
         bias = torch.empty(0)
         if cfg.alibi:
             self.past = S if first_pass else self.past + S
@@ -165,11 +166,13 @@ class Int8Decoder:
         for attn, ffn in self.layers:
             x = attn.forward(x, pad, self.reorder_state, True, True, first_pass, bias)
             x = ffn.forward(x, True, True)
-        return self.final_norm.layer_norm(x)
+        return ops._timed("final_rmsnorm", 2 * B * S * cfg.hidden * 2, lambda: self.final_norm.layer_norm(x))
 
     def logits(self, input_ids, first_pass=True, attention_mask=None):
         h = self(input_ids, first_pass, attention_mask)
-        return torch.nn.functional.linear(h[:, -1:, :], self.lm_head)
+        B = h.shape[0]
+        return ops._timed("lm_head fp16 (torch)", self.lm_head.numel() * 2 + B * (self.cfg.hidden + self.cfg.vocab) * 2,
+                          lambda: torch.nn.functional.linear(h[:, -1:, :], self.lm_head))
 
     @torch.no_grad()
     def greedy(self, input_ids, max_new_tokens, attention_mask=None):

@@ -150,6 +150,48 @@ def _check_vec(name, v, N):
 EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 
 
+class LaunchTimer:
+    """Per-kernel timing of the decode path for a benchmark's breakdown: while one is installed
+    (`ops.launch_timer = LaunchTimer()`), the incremental calls of the ops issue their launches
+    one library call at a time -- the same entry points with the same arguments that
+    eet_mmha_int8_decode / eet_gated_ffn_int8_decode issue from C++ -- each bracketed by a pair
+    of events on the current stream.  summary() waits for the GPU."""
+
+    def __init__(self):
+        self.records = []
+
+    def run(self, name, nbytes, fn):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        out = fn()
+        e1.record()
+        self.records.append((name, nbytes, e0, e1))
+        return out
+
+    def summary(self):
+        torch.cuda.synchronize()
+        agg = {}
+        for name, nbytes, e0, e1 in self.records:
+            a = agg.setdefault(name, [0, 0.0, 0])
+            a[0] += 1
+            a[1] += e0.elapsed_time(e1) * 1e3
+            a[2] += nbytes
+        return {k: {"calls": v[0], "us_total": v[1], "bytes_total": v[2]} for k, v in agg.items()}
+
+
+launch_timer = None
+
+
+def _timed(name, nbytes, fn):
+    return launch_timer.run(name, nbytes, fn) if launch_timer is not None else fn()
+
+
+def linear_bytes(M, K, N, epilogue=EPI_NONE):
+    """Algorithmic bytes of one int8 linear: every operand once."""
+    n_out = N // 2 if epilogue == EPI_SWIGLU else N
+    return K * N + 2 * N + 2 * M * K + 2 * M * n_out + (2 * M * N if epilogue == EPI_RESIDUAL else 0)
+
+
 RMS_FUSE_MAX_M = 32     # the RMSnorm prologue exists in the small-M kernel only
 
 
@@ -320,6 +362,19 @@ class _MmhaInt8:
             need = L.eet_mmha_int8_decode_workspace(B, H, dh, self.step)
             ws = workspaces.get("mmha_ws", max(need // 4, 1), torch.float32, dev)
             rope = self.rope_table.data_ptr() + (self.step - 1) * dh * 4 if self._rope else None
+            if launch_timer is not None:
+                inner, base = self.inner, qkv.data_ptr()
+                _timed("qkv_gemm+rmsnorm", linear_bytes(B, hidden, 3 * inner), lambda: _gemm(
+                    x, self.qkv_w, self.qkv_s, qkv, B, 3 * inner, hidden, EPI_NONE, None, self.gamma, desc.layernorm_eps))
+                attn_bytes = 2 * self.step * B * inner * 2 + 6 * B * inner * 2 + (2 * H * self.step if alibi is not None else 0)
+                _timed("decode_attention", attn_bytes, lambda: check(L.eet_mmha_decode(
+                    base, base + 2 * inner, base + 4 * inner, 3 * inner, self.k_cache.data_ptr(), self.v_cache.data_ptr(),
+                    cbuf.data_ptr(), _ptr(alibi), _ptr(pad), B, H, dh, self.step, self.t_cap, rope, ws.data_ptr(),
+                    ws.numel() * 4, _stream()), "eet_mmha_decode"))
+                _timed("o_gemm+residual", linear_bytes(B, inner, hidden, EPI_RESIDUAL), lambda: _gemm(
+                    cbuf, self.o_w, self.o_s, out, B, hidden, inner, EPI_RESIDUAL, x))
+                self._keep = (x, pad, alibi, reorder)
+                return out[: M * hidden].view(B, S, hidden)
             check(L.eet_mmha_int8_decode(x.data_ptr(), self.gamma.data_ptr(), desc.layernorm_eps,
                                          self.qkv_w.data_ptr(), self.qkv_s.data_ptr(), self.o_w.data_ptr(),
                                          self.o_s.data_ptr(), self.k_cache.data_ptr(), self.v_cache.data_ptr(),
@@ -444,6 +499,14 @@ class GatedFeedForwardNetworkInt8:
         out = workspaces.get(self.cache_name, cap * hidden, f16, dev)
         # fc1, fc2 and gated_act (gated_ffn_int8.cpp:253-301, 168-179) in one launch; at decode
         # sizes the RMSnorm (:112) rides in the same launch and fc3 follows from the same library call
+        if M <= RMS_FUSE_MAX_M and launch_timer is not None:
+            _timed("gate_up_gemm+rmsnorm+swiglu", linear_bytes(M, hidden, 2 * self.d_ff, EPI_SWIGLU), lambda: _gemm(
+                x, self.w01, self.s01, act, M, 2 * self.d_ff, hidden, EPI_SWIGLU, None, self.gamma, desc.layernorm_eps))
+            epi = EPI_RESIDUAL if add_residual else EPI_NONE
+            _timed("down_gemm+residual", linear_bytes(M, self.d_ff, hidden, epi), lambda: _gemm(
+                act, self.w2, self.s2, out, M, hidden, self.d_ff, epi, x if add_residual else None))
+            self._keep = x
+            return out[: M * hidden].view(B, S, hidden)
         if M <= RMS_FUSE_MAX_M:
             check(lib().eet_gated_ffn_int8_decode(x.data_ptr(), self.gamma.data_ptr(), desc.layernorm_eps,
                                                   self.w01.data_ptr(), self.s01.data_ptr(), self.w2.data_ptr(),

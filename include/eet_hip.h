@@ -269,6 +269,16 @@ int eet_prefill_attention(const void *q, const void *k_cache, const void *v_cach
                           const void *alibi, const int64_t *pad, int B, int H, int S, int dh,
                           int T_cap, void *stream);
 
+/* Measurement utility (no counterpart in the reference): reads `bytes` of device
+ * memory once with the access pattern and launch structure of the small-M GEMM
+ * (contiguous range per workgroup, 128-bit non-temporal loads, one reduction and
+ * one small store per workgroup) and nothing else.  Launched over the same
+ * buffers, in the same order and with the same grids as a GEMM pass, it measures
+ * the HBM rate this machine allows such a chain of dependent launches.  sink: 1 KiB
+ * of device memory per workgroup. */
+int eet_hbm_stream_probe(const void *src, size_t bytes, int workgroups, void *sink,
+                         size_t sink_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -300,7 +300,7 @@ def packer_bench(torch, eet):
     return out
 
 
-def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed, model=LLAMA):
+def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed, model=LLAMA, graph_batch1=True):
     """Int8 decoder of the given shape, random init: prefill `prompt` tokens then
     greedy-decode `gen` tokens; tokens/s = batch * (gen - 1) / decode time."""
     from eet_amd import decoder as D
@@ -357,6 +357,33 @@ def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed, model=LLAMA
         finally:
             _ops.launch_timer = None
         raw = timer.summary() if bd_steps else {}
+
+        # the same decode from HIP-graph replays of the incremental step, and both ways at batch 1
+        def timed_decode(b, graph):
+            lg = model.logits(ids[:b], True)
+            tok = torch.argmax(lg[:, -1, :], dim=-1)
+            if graph:
+                replay = model.capture_decode_step(tok)
+                replay()
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                for _ in range(gen - 1):
+                    replay()
+            else:
+                lg = model.logits(tok[:, None], False)
+                tok = torch.argmax(lg[:, -1, :], dim=-1)
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                for _ in range(gen - 1):
+                    lg = model.logits(tok[:, None], False)
+                    tok = torch.argmax(lg[:, -1, :], dim=-1)
+            torch.cuda.synchronize()
+            el = time.perf_counter() - t
+            return {"tokens_per_s": round(b * (gen - 1) / el, 1), "ms_per_token_step": round(el / (gen - 1) * 1e3, 3)}
+        eager_vs_graph = {f"batch {batch} graph": timed_decode(batch, True)}
+        if graph_batch1:
+            eager_vs_graph["batch 1 eager"] = timed_decode(1, False)
+            eager_vs_graph["batch 1 graph"] = timed_decode(1, True)
     steps = gen - 1
     ms = t_dec / steps * 1e3
     # A bracket (event, launch, event) costs more than the launch does back to back -- the two event
@@ -382,6 +409,7 @@ def decode_bench(torch, eet, weights, dev, batch, prompt, gen, seed, model=LLAMA
             "prompt": prompt, "generated": gen, "layers": len(weights), "prefill_s": round(t_prefill, 3), "prefill_warm_s": round(t_prefill_warm, 3),
             "step_hbm_bytes": step_bytes,
             "step_roofline_frac": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "hip_graph_replay": eager_vs_graph,
             "breakdown": breakdown,
             "breakdown_note": f"{bd_steps} further token steps with every launch issued on its own between two events; "
                               "us_per_call is the bracketed time scaled so that the kernels of a step sum to "
@@ -660,7 +688,8 @@ def main():
         _ops.workspaces.clear()
         _ops.spare_kv.clear()
         bw = make_weights(torch, eet, dev, BAICHUAN13B["layers"], BAICHUAN13B["hidden"], BAICHUAN13B["d_ff"], seed=4321)
-        result["decode_baichuan13b"] = decode_bench(torch, eet, bw, dev, 32, 2048, 256, seed=9, model=BAICHUAN13B)
+        result["decode_baichuan13b"] = decode_bench(torch, eet, bw, dev, 32, 2048, 256, seed=9, model=BAICHUAN13B,
+                                                    graph_batch1=False)
         del bw
 
     if not args.no_cpu:

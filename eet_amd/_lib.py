@@ -31,6 +31,12 @@ SIGNATURES = {
     "eet_mmha_decode": (_i, [_vp, _vp, _vp, _l, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
     "eet_mmha_decode_static_capacity": (_sz, []),
     "eet_mmha_decode_static": (_i, [_vp, _vp, _vp, _l, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp]),
+    "eet_step_advance": (_i, [_vp, _i, _vp]),
+    "eet_mmha_decode_replayable_workspace": (_sz, [_i, _i, _i, _i]),
+    "eet_mmha_decode_replayable": (_i, [_vp, _vp, _vp, _l, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp, _i, _i, _vp, _vp,
+                                        _sz, _vp]),
+    "eet_mmha_int8_decode_replayable": (_i, [_vp, _vp, _f] + [_vp] * 7 + [_i] + [_vp] * 5 + [_i] * 4 + [_vp, _i, _i, _vp,
+                                                                                                 _sz, _vp]),
     "eet_mmha_int8_decode_workspace": (_sz, [_i, _i, _i, _i]),
     "eet_mmha_int8_decode": (_i, [_vp, _vp, _f] + [_vp] * 12 + [_i] * 6 + [_vp, _sz, _vp]),
     "eet_gated_ffn_int8_decode": (_i, [_vp, _vp, _f] + [_vp] * 6 + [_i] * 4 + [_vp]),

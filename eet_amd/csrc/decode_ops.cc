@@ -89,3 +89,37 @@ extern "C" int eet_gated_ffn_int8_decode(const void *x, const void *rms_gamma, f
                                 add_residual ? EET_EPILOGUE_RESIDUAL : EET_EPILOGUE_NONE, add_residual ? x : nullptr,
                                 nullptr, 0.f, nullptr, 0, stream);
 }
+
+// The same incremental call in its replayable form (see eet_mmha_decode_replayable): recorded once
+// into a HIP graph, it serves every later token.
+extern "C" int eet_mmha_int8_decode_replayable(const void *x, const void *rms_gamma, float rms_eps, const void *qkv_w,
+                                               const void *qkv_scale, const void *o_w, const void *o_scale,
+                                               void *k_cache, void *v_cache, const void *alibi, int alibi_ld,
+                                               const int64_t *pad, const float *rope_table, void *qkv_buf,
+                                               void *ctx_buf, void *out, int B, int H, int dh, int hidden,
+                                               const int *step_dev, int step_max, int T_cap, void *workspace,
+                                               size_t workspace_bytes, void *stream)
+{
+    EET_REQUIRE(x && rms_gamma && qkv_buf && ctx_buf && out, EET_ERR_INVALID_ARGUMENT,
+                "eet_mmha_int8_decode_replayable: null pointer");
+    EET_REQUIRE(B > 0 && B <= 32 && H > 0 && dh > 0 && hidden > 0, EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_mmha_int8_decode_replayable: B=%d must be 1..32 (one token per sequence), H=%d dh=%d hidden=%d", B,
+                H, dh, hidden);
+    const int inner = H * dh;
+    {
+        const size_t xb = (size_t)B * hidden * 2, qb = (size_t)B * 3 * inner * 2, cb = (size_t)B * inner * 2;
+        EET_REQUIRE(!overlaps(out, xb, x, xb) && !overlaps(qkv_buf, qb, x, xb) && !overlaps(ctx_buf, cb, x, xb) &&
+                        !overlaps(ctx_buf, cb, qkv_buf, qb) && !overlaps(out, xb, ctx_buf, cb),
+                    EET_ERR_INVALID_ARGUMENT, "eet_mmha_int8_decode_replayable: x, qkv_buf, ctx_buf and out must not overlap");
+    }
+    if (int rc = eet_gemm_w8a16_fused(x, qkv_w, qkv_scale, qkv_buf, B, 3 * inner, hidden, EET_EPILOGUE_NONE, nullptr,
+                                      rms_gamma, rms_eps, nullptr, 0, stream))
+        return rc;
+    const _Float16 *base = static_cast<const _Float16 *>(qkv_buf);
+    if (int rc = eet_mmha_decode_replayable(base, base + inner, base + 2 * inner, 3L * inner, k_cache, v_cache, ctx_buf,
+                                            alibi, alibi_ld, pad, B, H, dh, step_dev, step_max, T_cap, rope_table,
+                                            workspace, workspace_bytes, stream))
+        return rc;
+    return eet_gemm_w8a16_fused(ctx_buf, o_w, o_scale, out, B, hidden, inner, EET_EPILOGUE_RESIDUAL, x, nullptr, 0.f,
+                                nullptr, 0, stream);
+}

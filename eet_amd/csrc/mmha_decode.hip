@@ -84,8 +84,17 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_new, const _Float16 *__restrict__ v_new,
     long qkv_stride, _Float16 *__restrict__ k_cache, _Float16 *__restrict__ v_cache, _Float16 *__restrict__ ctx,
     const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, float *__restrict__ partial, int H,
-    int step, int T_cap, int nsplit, float scale, const float *__restrict__ rope_row)
+    int step, int T_cap, int nsplit, float scale, const float *__restrict__ rope_row,
+    const int *__restrict__ step_dev, int alibi_ld_arg)
 {
+    // Replayable form (a launch recorded into a HIP graph): the step lives in device
+    // memory, rope_row is the base of the whole rotary table and the bias rows have a
+    // fixed leading dimension, so that the same recorded arguments serve every step.
+    if (step_dev != nullptr) {
+        step = min(max(*step_dev, 1), T_cap);
+        if (rope_row != nullptr)
+            rope_row += (size_t)(step - 1) * DH;
+    }
     constexpr int LPR = lanes_per_row(DH);   // lanes per row
     constexpr int NS = slices_per_row(DH);   // of which this many hold a slice
     constexpr int RPB = THREADS / LPR;       // row streams of the block (one per group of LPR lanes)
@@ -94,7 +103,7 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
 
     const int split = blockIdx.y;
     const int bh = blockIdx.x;
-    const int alibi_ld = step;
+    const int alibi_ld = alibi_ld_arg > 0 ? alibi_ld_arg : step;
     const int b = bh / H, h = bh % H;
     const int tid = threadIdx.x;
     const int sub = tid % LPR;   // which 8-element slice of the row
@@ -355,7 +364,7 @@ Plan pick_plan(int BH, int dh, int step)
 template <int DH, int THREADS>
 int launch_split(const void *q, const void *k, const void *v, long qkv_stride, void *kc, void *vc, void *ctx,
                  const void *alibi, const int64_t *pad, int B, int H, int step, int T_cap, void *ws, Plan plan,
-                 const float *rope_row, hipStream_t st)
+                 const float *rope_row, hipStream_t st, const int *step_dev = nullptr, int alibi_ld = 0)
 {
     const float scale = (float)(_Float16)(1.0f / sqrtf((float)DH));
     const int nsplit = plan.nsplit;
@@ -368,7 +377,7 @@ int launch_split(const void *q, const void *k, const void *v, long qkv_stride, v
                        static_cast<const _Float16 *>(v), qkv_stride, static_cast<_Float16 *>(kc),
                        static_cast<_Float16 *>(vc), static_cast<_Float16 *>(ctx),
                        static_cast<const _Float16 *>(alibi), pad, static_cast<float *>(ws), H, step, T_cap, nsplit,
-                       scale, rope_row);
+                       scale, rope_row, step_dev, alibi_ld);
     EET_HIP_CHECK(hipGetLastError());
     if (nsplit > 1) {
         hipLaunchKernelGGL((mmha_decode_merge_kernel<DH>), dim3(B * H), dim3(DH), 0, st,
@@ -381,16 +390,16 @@ int launch_split(const void *q, const void *k, const void *v, long qkv_stride, v
 template <int DH>
 int launch(const void *q, const void *k, const void *v, long qkv_stride, void *kc, void *vc, void *ctx,
            const void *alibi, const int64_t *pad, int B, int H, int step, int T_cap, void *ws, Plan plan,
-           const float *rope_row, hipStream_t st)
+           const float *rope_row, hipStream_t st, const int *step_dev = nullptr, int alibi_ld = 0)
 {
     if (plan.threads == 1024)
         return launch_split<DH, 1024>(q, k, v, qkv_stride, kc, vc, ctx, alibi, pad, B, H, step, T_cap, ws, plan,
-                                      rope_row, st);
+                                      rope_row, st, step_dev, alibi_ld);
     if (plan.threads == 512)
         return launch_split<DH, 512>(q, k, v, qkv_stride, kc, vc, ctx, alibi, pad, B, H, step, T_cap, ws, plan,
-                                     rope_row, st);
+                                     rope_row, st, step_dev, alibi_ld);
     return launch_split<DH, 256>(q, k, v, qkv_stride, kc, vc, ctx, alibi, pad, B, H, step, T_cap, ws, plan, rope_row,
-                                 st);
+                                 st, step_dev, alibi_ld);
 }
 
 }  // namespace
@@ -452,21 +461,22 @@ static int check_mmha_args(const char *fn, const void *q, const void *k, const v
 
 static int run_mmha(const void *q, const void *k, const void *v, long qkv_stride, void *k_cache, void *v_cache,
                     void *ctx, const void *alibi, const int64_t *pad, int B, int H, int dh, int step, int T_cap,
-                    const float *rope_cos_sin, void *partials, Plan plan, hipStream_t st)
+                    const float *rope_cos_sin, void *partials, Plan plan, hipStream_t st,
+                    const int *step_dev = nullptr, int alibi_ld = 0)
 {
     switch (dh) {
         case 32:
             return launch<32>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, partials,
-                              plan, rope_cos_sin, st);
+                              plan, rope_cos_sin, st, step_dev, alibi_ld);
         case 64:
             return launch<64>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, partials,
-                              plan, rope_cos_sin, st);
+                              plan, rope_cos_sin, st, step_dev, alibi_ld);
         case 96:
             return launch<96>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, partials,
-                              plan, rope_cos_sin, st);
+                              plan, rope_cos_sin, st, step_dev, alibi_ld);
         default:
             return launch<128>(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, step, T_cap, partials,
-                               plan, rope_cos_sin, st);
+                               plan, rope_cos_sin, st, step_dev, alibi_ld);
     }
 }
 
@@ -484,6 +494,49 @@ extern "C" int eet_mmha_decode(const void *q, const void *k, const void *v, long
                 "eet_mmha_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     return run_mmha(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, dh, step, T_cap, rope_cos_sin,
                     workspace, plan, static_cast<hipStream_t>(stream));
+}
+
+// ---------------------------------------------------------------------------
+// Replayable form: the step comes from device memory, so the launch can be
+// recorded once into a HIP graph and replayed for every token.
+// ---------------------------------------------------------------------------
+namespace {
+__global__ void step_advance_kernel(int *step, int by) { *step += by; }
+}  // namespace
+
+extern "C" int eet_step_advance(int *step_dev, int by, void *stream)
+{
+    EET_REQUIRE(step_dev != nullptr, EET_ERR_INVALID_ARGUMENT, "eet_step_advance: null pointer");
+    hipLaunchKernelGGL(step_advance_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), step_dev, by);
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
+extern "C" size_t eet_mmha_decode_replayable_workspace(int B, int H, int dh, int step_max)
+{
+    return eet_mmha_decode_workspace(B, H, dh, step_max);
+}
+
+extern "C" int eet_mmha_decode_replayable(const void *q, const void *k, const void *v, long qkv_stride, void *k_cache,
+                                          void *v_cache, void *ctx, const void *alibi, int alibi_ld, const int64_t *pad,
+                                          int B, int H, int dh, const int *step_dev, int step_max, int T_cap,
+                                          const float *rope_table, void *workspace, size_t workspace_bytes,
+                                          void *stream)
+{
+    EET_REQUIRE(step_dev != nullptr, EET_ERR_INVALID_ARGUMENT, "eet_mmha_decode_replayable: null step pointer");
+    EET_REQUIRE(alibi == nullptr || alibi_ld >= step_max, EET_ERR_INVALID_ARGUMENT,
+                "eet_mmha_decode_replayable: the bias rows need a leading dimension of at least step_max (%d), got %d",
+                step_max, alibi_ld);
+    Plan plan;
+    if (int rc = check_mmha_args("eet_mmha_decode_replayable", q, k, v, qkv_stride, k_cache, v_cache, ctx, B, H, dh,
+                                 step_max, T_cap, rope_table, &plan))
+        return rc;
+    const size_t need = plan.nsplit > 1 ? (size_t)B * H * plan.nsplit * (dh + 2) * sizeof(float) : 0;
+    EET_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), EET_ERR_WORKSPACE,
+                "eet_mmha_decode_replayable: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    // the launch shape is that of step_max; the kernel reads the step of each replay itself
+    return run_mmha(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, dh, step_max, T_cap, rope_table,
+                    workspace, plan, static_cast<hipStream_t>(stream), step_dev, alibi_ld);
 }
 
 // ---------------------------------------------------------------------------

@@ -145,6 +145,8 @@ class Int8Decoder:
         if first_pass:
             # the op reads the last row of the [H, S, S] mask; hand it that row as a [H, 1->S, S] view
             return self._mask[:, None, :L].expand(cfg.heads, L, L)
+        if ops.replay_state is not None:
+            return self._mask[:, None, :]         # the whole table: the kernel reads the step itself
         return self._mask[:, None, :L].contiguous()
 
     def __call__(self, input_ids, first_pass=True, attention_mask=None):
@@ -185,4 +187,72 @@ class Int8Decoder:
             out.append(nxt)
             if i + 1 < max_new_tokens:
                 logits = self.logits(nxt[:, None], False, attention_mask)
+        return torch.stack(out, dim=1)
+
+    # ---- the incremental step as a HIP graph ---------------------------------------------------
+    def _shift_host_steps(self, by):
+        for attn, _ in self.layers:
+            attn.step += by
+        if self.cfg.alibi:
+            self.past += by
+
+    def capture_decode_step(self, next_ids):
+        """Records one incremental step (step counter advance, embedding, all layers, final norm,
+        lm_head, argmax, feeding the token back) into a HIP graph, after a prompt has been
+        processed eagerly.  next_ids [B] are the tokens the first replay consumes.  Returns a
+        function that replays the step and returns the new tokens [B] (a static buffer)."""
+        cfg, dev = self.cfg, self.embed.device
+        B = next_ids.shape[0]
+        lib = ops.lib()
+        step_dev = torch.tensor([self.layers[0][0].step], dtype=torch.int32, device=dev)
+        ids = next_ids.reshape(B, 1).clone()
+        out_tok = torch.zeros(B, dtype=torch.long, device=dev)
+        ops.replay_state = ops.ReplayState(step_dev, cfg.max_full_seq)
+
+        def one_step():
+            ops.check(lib.eet_step_advance(step_dev.data_ptr(), 1, ops._stream()), "eet_step_advance")
+            logits = self.logits(ids, False)
+            out_tok.copy_(torch.argmax(logits[:, -1, :], dim=-1))
+            ids.copy_(out_tok[:, None])
+        try:
+            # eager warm-up on a side stream (allocates every workspace), then undone: the cache row it
+            # wrote is written again by the first replay
+            keep = ids.clone()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side), torch.no_grad():
+                one_step()
+                ops.check(lib.eet_step_advance(step_dev.data_ptr(), -1, ops._stream()), "eet_step_advance")
+                ids.copy_(keep)
+            torch.cuda.current_stream().wait_stream(side)
+            self._shift_host_steps(-1)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph), torch.no_grad():
+                one_step()
+            self._shift_host_steps(-1)      # recording ran the host code once; no kernel has run
+        finally:
+            ops.replay_state = None
+
+        def replay():
+            if self.layers[0][0].step + 1 > cfg.max_full_seq:
+                raise RuntimeError(f"[EET][ERROR] decode step {self.layers[0][0].step + 1} exceeds max_full_seq "
+                                   f"{cfg.max_full_seq}")
+            graph.replay()
+            self._shift_host_steps(1)
+            return out_tok
+        self._graph_keep = (graph, step_dev, ids, out_tok)
+        return replay
+
+    @torch.no_grad()
+    def greedy_graph(self, input_ids, max_new_tokens, attention_mask=None):
+        """greedy() with the incremental step replayed from a HIP graph."""
+        logits = self.logits(input_ids, True, attention_mask)
+        nxt = torch.argmax(logits[:, -1, :], dim=-1)
+        out = [nxt]
+        if max_new_tokens > 1:
+            if attention_mask is not None:
+                raise NotImplementedError("greedy_graph: left-padded batches run through greedy()")
+            replay = self.capture_decode_step(nxt)
+            for _ in range(max_new_tokens - 1):
+                out.append(replay().clone())
         return torch.stack(out, dim=1)

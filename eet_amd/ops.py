@@ -182,6 +182,18 @@ class LaunchTimer:
 launch_timer = None
 
 
+class ReplayState:
+    """Set as `ops.replay_state` while a decoder records its incremental step into a HIP graph (and
+    for the eager warm-up before it): the attention ops then issue the replayable form of their
+    call, which reads the step from `step_dev` (int32 on the GPU) instead of taking it by value."""
+
+    def __init__(self, step_dev, step_max):
+        self.step_dev, self.step_max = step_dev, int(step_max)
+
+
+replay_state = None
+
+
 def _timed(name, nbytes, fn):
     return launch_timer.run(name, nbytes, fn) if launch_timer is not None else fn()
 
@@ -354,13 +366,34 @@ class _MmhaInt8:
             # the whole incremental call from one library call: RMSnorm + QKV, rotary + append +
             # attention, output projection + residual
             alibi = None
-            if bias is not None:
+            if bias is not None and replay_state is None:
                 if bias.numel() != H * self.step:
                     raise RuntimeError(f"[EET][ERROR] {self._name}: relative_attention_bias must be [H, 1, step] "
                                        f"with step={self.step}, got {tuple(bias.shape)}")
                 alibi = bias.to(f16).contiguous()
             need = L.eet_mmha_int8_decode_workspace(B, H, dh, self.step)
             ws = workspaces.get("mmha_ws", max(need // 4, 1), torch.float32, dev)
+            if replay_state is not None:
+                rs = replay_state
+                ld = 0
+                if bias is not None:
+                    # the whole [H, T] table with a fixed leading dimension: the kernel reads row entries < step
+                    ld = bias.shape[-1]
+                    if bias.numel() != H * ld or ld < rs.step_max:
+                        raise RuntimeError(f"[EET][ERROR] {self._name}: a replayable step needs the bias table "
+                                           f"[H, >= {rs.step_max}], got {tuple(bias.shape)}")
+                    alibi = bias.to(f16).contiguous()
+                need = L.eet_mmha_decode_replayable_workspace(B, H, dh, rs.step_max)
+                ws = workspaces.get("mmha_ws", max(need // 4, 1), torch.float32, dev)
+                check(L.eet_mmha_int8_decode_replayable(
+                    x.data_ptr(), self.gamma.data_ptr(), desc.layernorm_eps, self.qkv_w.data_ptr(),
+                    self.qkv_s.data_ptr(), self.o_w.data_ptr(), self.o_s.data_ptr(), self.k_cache.data_ptr(),
+                    self.v_cache.data_ptr(), _ptr(alibi), ld, _ptr(pad),
+                    self.rope_table.data_ptr() if self._rope else None, qkv.data_ptr(), cbuf.data_ptr(), out.data_ptr(),
+                    B, H, dh, hidden, rs.step_dev.data_ptr(), rs.step_max, self.t_cap, ws.data_ptr(), ws.numel() * 4,
+                    _stream()), "eet_mmha_int8_decode_replayable")
+                self._keep = (x, pad, alibi, reorder)
+                return out[: M * hidden].view(B, S, hidden)
             rope = self.rope_table.data_ptr() + (self.step - 1) * dh * 4 if self._rope else None
             if launch_timer is not None:
                 inner, base = self.inner, qkv.data_ptr()

@@ -269,6 +269,37 @@ int eet_prefill_attention(const void *q, const void *k_cache, const void *v_cach
                           const void *alibi, const int64_t *pad, int B, int H, int S, int dh,
                           int T_cap, void *stream);
 
+/* Replayable forms of the incremental attention call, for a decode step that is
+ * recorded once into a HIP graph and replayed for every token (the reference
+ * re-issues the launch sequence of csrc/op/llama_mmha.cpp:202-266 from the host
+ * for every token).  What changes from step to step lives in device memory:
+ *   step_dev    int32 in device memory: the step of this call (rows attended,
+ *               the new token included); eet_step_advance(step_dev, 1, stream)
+ *               recorded ahead of the layers moves it on at each replay
+ *   step_max    the largest step the recording will be replayed at (<= T_cap):
+ *               launch shape and workspace are chosen for it
+ *   rope_table  NULL or the BASE of the eet_rope_table table (>= step_max rows):
+ *               the kernel picks row step-1 itself
+ *   alibi       NULL or [H][alibi_ld] half with alibi_ld >= step_max
+ * Everything else is as in eet_mmha_decode / eet_mmha_int8_decode; results are
+ * bit-identical to those calls at the same step when the launch shapes agree. */
+int eet_step_advance(int *step_dev, int by, void *stream);
+size_t eet_mmha_decode_replayable_workspace(int B, int H, int dh, int step_max);
+int eet_mmha_decode_replayable(const void *q, const void *k, const void *v, long qkv_stride,
+                               void *k_cache, void *v_cache, void *ctx, const void *alibi,
+                               int alibi_ld, const int64_t *pad, int B, int H, int dh,
+                               const int *step_dev, int step_max, int T_cap,
+                               const float *rope_table, void *workspace, size_t workspace_bytes,
+                               void *stream);
+int eet_mmha_int8_decode_replayable(const void *x, const void *rms_gamma, float rms_eps,
+                                    const void *qkv_w, const void *qkv_scale, const void *o_w,
+                                    const void *o_scale, void *k_cache, void *v_cache,
+                                    const void *alibi, int alibi_ld, const int64_t *pad,
+                                    const float *rope_table, void *qkv_buf, void *ctx_buf, void *out,
+                                    int B, int H, int dh, int hidden, const int *step_dev,
+                                    int step_max, int T_cap, void *workspace, size_t workspace_bytes,
+                                    void *stream);
+
 /* Measurement utility (no counterpart in the reference): reads `bytes` of device
  * memory once with the access pattern and launch structure of the small-M GEMM
  * (contiguous range per workgroup, 128-bit non-temporal loads, one reduction and

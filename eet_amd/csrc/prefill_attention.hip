@@ -29,8 +29,10 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <type_traits>
 
 #include "common.h"
+#include "tuning.h"
 
 namespace {
 
@@ -297,6 +299,320 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 #endif
 }
 
+
+// ---------------------------------------------------------------------------
+// Head size 128 (LLaMA-7B, Baichuan-13B): the same transposed formulation with
+// the K and V chunks brought into LDS by the memory pipeline itself.
+//
+// A workgroup of 8 wavefronts takes 256 queries of one (b, h); wavefront w owns
+// the 16-query tiles w and w + 8 of the block (one early, one late, so that the
+// causal triangle is split evenly) and skips a tile once the chunks have passed
+// its diagonal.  K and V rows stay row-major in LDS, 256 B per row, copied
+// global -> LDS with buffer_load_dwordx4 ... lds (no staging registers, no
+// ds_write) into a ring of four 64-key stages, one pair of chunks ahead of the
+// pair being multiplied; one s_barrier per pair.  Piece p (16 B) of row r sits at
+// position p ^ swz(r), with one swizzle for K and another for V, so that the K
+// operand reads (lane = row) and the V reads hit distinct banks.  V^T operands come out of the row-major rows through
+// ds_read_b64_tr_b16, which hands lane i column i of a 4 x 16 block of halves.
+// ---------------------------------------------------------------------------
+constexpr int kD = 128;
+constexpr int kWaves2 = 8, kBQ2 = 256, kStages = 4;
+constexpr int kStageVec = 2 * 1024 + 16;   // u32x4 per stage: K rows, V rows, bias row (+ padding)
+
+// Measured on MI355X with 8 wavefronts reading back to back: a 16-byte operand read (lane = row) runs at
+// full rate when the piece index is XORed with the row number itself, and at half rate with the V
+// swizzle or with rows padded to 272 B; the transposing 8-byte reads of V run at full rate with the
+// swizzle below (4 consecutive rows must land on 4 different pairs of positions) and not with padding.
+__device__ __forceinline__ int k_swz(int r) { return r & 15; }
+__device__ __forceinline__ int row_swz(int r) { return ((r & 7) << 1) | ((r >> 3) & 1); }
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+template <bool ALIBI>
+__global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attention_dh128_kernel(
+    const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_cache, const _Float16 *__restrict__ v_cache,
+    _Float16 *__restrict__ ctx, const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, int H, int S,
+    int T_cap, float scale)
+{
+#if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
+    constexpr int DC = kD / 32, DT = kD / 16;
+    __shared__ u32x4 lds[kStages * kStageVec];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, j = lane & 15;
+    const int bh = blockIdx.y, b = bh / H, h = bh % H;
+    const int q_blocks = (S + kBQ2 - 1) / kBQ2;
+    const int q0 = (q_blocks - 1 - (int)blockIdx.x) * kBQ2;  // late (long) query blocks first
+    const int padb = pad ? (int)min((int64_t)S, max((int64_t)0, pad[b])) : 0;
+
+    const _Float16 *kbase = k_cache + (size_t)bh * T_cap * kD;
+    const _Float16 *vbase = v_cache + (size_t)bh * T_cap * kD;
+    const _Float16 *qbase = q + (size_t)bh * S * kD;
+    // rows >= S are out of range: they read as zeros (and are masked: such a key follows every query)
+    const __amdgpu_buffer_rsrc_t krs =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16 *>(kbase), 0, (unsigned)S * (kD * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrs =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16 *>(vbase), 0, (unsigned)S * (kD * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t ars = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<_Float16 *>(ALIBI ? alibi + (size_t)h * S : q), 0, ALIBI ? (unsigned)S * 2u : 0u, 0x00020000);
+
+    // the two query tiles of this wavefront
+    int tq0[2] = {q0 + 16 * wave, q0 + 16 * (wave + kWaves2)};
+    half8 qop[2][DC];
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        const int qi = min(tq0[qt] + j, S - 1);
+#pragma unroll
+        for (int c = 0; c < DC; ++c)
+            qop[qt][c] = *reinterpret_cast<const half8 *>(qbase + (size_t)qi * kD + 32 * c + 8 * g);
+    }
+    floatx4 oacc[2][DT];
+    float m_run[2], l_run[2];
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        m_run[qt] = -INFINITY;
+        l_run[qt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            oacc[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // DMA: instruction t of a chunk fills rows 4t .. 4t+3 (1 KiB); lane l carries position l % 16 of row
+    // 4t + l / 16, i.e. piece (l % 16) ^ swz(row).  Wavefront w issues instructions 2w and 2w + 1 of K and of V.
+    int dma_off_k[2], dma_off_v[2];   // byte offset of this lane's piece within a chunk, for its two instructions
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int row = 4 * (2 * wave + i) + (lane >> 4);
+        dma_off_k[i] = row * (kD * 2) + (((lane & 15) ^ k_swz(row)) << 4);
+        dma_off_v[i] = row * (kD * 2) + (((lane & 15) ^ row_swz(row)) << 4);
+    }
+    auto dma_chunk = [&](int stage, int kc0) {
+        u32x4 *st = lds + stage * kStageVec;
+        const int base = kc0 * (kD * 2);   // in the lane offset: the range check of a buffer load covers it
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(krs, st + (2 * wave + i) * 64, 16, base + dma_off_k[i], 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(vrs, st + 1024 + (2 * wave + i) * 64, 16, base + dma_off_v[i], 0, 0, 0);
+        }
+        if (ALIBI)   // the chunk's 64 bias terms (128 B): every wavefront writes the same bytes
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ars, st + 2048, 4, kc0 * 2 + (lane & 31) * 4, 0, 0, 0);
+    };
+
+    constexpr float kLog2e = 1.4426950408889634f;
+    const float scale2 = scale * kLog2e;
+    const int k_begin = (padb / kBK) * kBK;
+    const int k_end = min(S, q0 + kBQ2);
+    const int nchunks = (k_end - k_begin + kBK - 1) / kBK;
+
+    // the work on one chunk for the query tiles named in MASK (bit qt)
+    auto compute = [&](auto mask_c, const u32x4 *st, int kc0) {
+        constexpr int MASK = decltype(mask_c)::value;
+        const u32x4 *kst = st;
+        const unsigned char *vst = reinterpret_cast<const unsigned char *>(st + 1024);
+        floatx4 sacc[2][4];
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+                sacc[qt][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            const int row = 16 * kt + j;
+#pragma unroll
+            for (int c = 0; c < DC; ++c) {
+                const half8 kop = __builtin_bit_cast(half8, kst[row * 16 + ((4 * c + g) ^ k_swz(row))]);
+#pragma unroll
+                for (int qt = 0; qt < 2; ++qt)
+                    if (MASK & (1 << qt))
+                        sacc[qt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop, qop[qt][c], sacc[qt][kt], 0, 0, 0);
+            }
+        }
+        // operand reads three ahead of the matrix instructions that use them
+        {
+            constexpr int kPer = (MASK == 3) ? 2 : 1;
+            __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+#pragma unroll
+            for (int n = 0; n < 13; ++n) {
+                __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 3 * kPer, 0);
+        }
+        half4 bias4[4];
+        if (ALIBI) {
+            const _Float16 *bst = reinterpret_cast<const _Float16 *>(st + 2048);
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+                bias4[kt] = *reinterpret_cast<const half4 *>(bst + 16 * kt + 4 * g);
+        }
+        half8 pop[2][2];
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+            if (!(MASK & (1 << qt)))
+                continue;
+            const int qi = tq0[qt] + j;
+            float cmax = -INFINITY;
+            const bool need_mask = (kc0 + kBK - 1 > tq0[qt]) || (kc0 < padb);
+            // Without a bias the scale is applied inside the exponent's argument (one fused multiply-add per
+            // element instead of a multiply and a subtract): the maximum is taken over the raw products and
+            // scaled once (the scale is positive).
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float s = sacc[qt][kt][r];
+                    if (ALIBI)
+                        s = s * scale2 + (float)bias4[kt][r] * kLog2e;
+                    if (need_mask) {
+                        const int key = kc0 + 16 * kt + 4 * g + r;
+                        s = (key > qi || key < padb) ? -INFINITY : s;
+                    }
+                    sacc[qt][kt][r] = s;
+                    cmax = fmaxf(cmax, s);
+                }
+            cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
+            cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+            if (!ALIBI)
+                cmax *= scale2;
+            const float m_new = fmaxf(m_run[qt], cmax);
+            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+            const float corr = __builtin_amdgcn_exp2f(m_run[qt] - m_safe);  // 0 while nothing has been seen
+            float psum = 0.f;
+            float p[4][4];
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    p[kt][r] = ALIBI ? __builtin_amdgcn_exp2f(sacc[qt][kt][r] - m_safe)
+                                     : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qt][kt][r], scale2, -m_safe));
+                    psum += p[kt][r];
+                }
+            l_run[qt] = l_run[qt] * corr + psum;
+            m_run[qt] = m_new;
+            // the accumulator is rescaled only when some query's maximum moved (rare after the first chunks)
+            if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    oacc[qt][dt] *= corr;
+            }
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                half8 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    o[r] = (_Float16)p[2 * hf][r];
+                    o[4 + r] = (_Float16)p[2 * hf + 1][r];
+                }
+                pop[qt][hf] = o;
+            }
+        }
+        // O^T += V^T . P^T.  Lane (g, j) needs d = 16*dt + j and keys 4g .. 4g+3 of tiles 2*hf and 2*hf + 1.
+        // One transposing read covers the 4 keys of one tile: lane j of a 16-lane group supplies 8 bytes
+        // (d = 16*dt + 4*(j%4) .. +3) of key row 4g + j/4 and receives the column d = 16*dt + j.
+        const int vr = j >> 2, vc4 = j & 3;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                short4v part[2];
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    const int key = 32 * hf + 16 * a + 4 * g + vr;
+                    const int pos = (2 * dt + (vc4 >> 1)) ^ row_swz(key);
+                    const unsigned char *addr = vst + key * (kD * 2) + pos * 16 + (vc4 & 1) * 8;
+                    part[a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (short4v __attribute__((address_space(3))) *)(addr));
+                }
+                const half4 lo = __builtin_bit_cast(half4, part[0]), hi = __builtin_bit_cast(half4, part[1]);
+                const half8 vop = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+                for (int qt = 0; qt < 2; ++qt)
+                    if (MASK & (1 << qt))
+                        oacc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop, pop[qt][hf], oacc[qt][dt], 0, 0, 0);
+            }
+        }
+        // the transposing reads (two per operand) two operands ahead of the matrix instructions
+        {
+            constexpr int kPer = (MASK == 3) ? 2 : 1;
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+            for (int n = 0; n < 2 * DT - 2; ++n) {
+                __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 2 * kPer, 0);
+        }
+    };
+
+    auto chunk = [&](int c) {
+        const int kc0 = k_begin + c * kBK;
+        const u32x4 *st = lds + (c % kStages) * kStageVec;
+        const bool t0 = kc0 <= tq0[0] + 15 && tq0[0] < S, t1 = kc0 <= tq0[1] + 15 && tq0[1] < S;
+        if (t0 && t1)
+            compute(std::integral_constant<int, 3>{}, st, kc0);
+        else if (t1)
+            compute(std::integral_constant<int, 2>{}, st, kc0);
+        else if (t0)
+            compute(std::integral_constant<int, 1>{}, st, kc0);
+    };
+    // Two chunks per barrier: while chunks 2i and 2i + 1 are multiplied, 2i + 2 and 2i + 3 are on their way
+    // into the other two stages.  (A chunk past the end reads rows >= S: zeros, no memory touched beyond
+    // the range; past k_end but below S it is a wasted copy.)
+    dma_chunk(0, k_begin);
+    dma_chunk(1, k_begin + kBK);
+    for (int i = 0; 2 * i < nchunks; ++i) {
+        // everything requested so far is this iteration's pair of chunks
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+        dma_chunk((2 * i + 2) % kStages, k_begin + (2 * i + 2) * kBK);   // these two stages were read in iteration i - 1
+        dma_chunk((2 * i + 3) % kStages, k_begin + (2 * i + 3) * kBK);
+        chunk(2 * i);
+        if (2 * i + 1 < nchunks)
+            chunk(2 * i + 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no copy may land in LDS after the workgroup has gone
+
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        float l = l_run[qt];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        const int qi = tq0[qt] + j;
+        if (qi >= S)
+            continue;
+        const float inv = (qi < padb) ? 0.f : 1.0f / (l + 1e-6f);
+        _Float16 *dst = ctx + ((size_t)(b * S + qi) * H + h) * kD;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            half4 o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                o[r] = (_Float16)(oacc[qt][dt][r] * inv);
+            *reinterpret_cast<half4 *>(dst + 16 * dt + 4 * g) = o;
+        }
+    }
+#endif
+}
+
+int launch_dh128(const void *q, const void *kc, const void *vc, void *ctx, const void *alibi, const int64_t *pad, int B,
+                 int H, int S, int T_cap, hipStream_t st)
+{
+    const float scale = (float)(_Float16)(1.0f / sqrtf(128.0f));
+    dim3 grid((S + kBQ2 - 1) / kBQ2, B * H);
+    if (alibi != nullptr)
+        hipLaunchKernelGGL((prefill_attention_dh128_kernel<true>), grid, dim3(64 * kWaves2), 0, st,
+                           static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(kc),
+                           static_cast<const _Float16 *>(vc), static_cast<_Float16 *>(ctx),
+                           static_cast<const _Float16 *>(alibi), pad, H, S, T_cap, scale);
+    else
+        hipLaunchKernelGGL((prefill_attention_dh128_kernel<false>), grid, dim3(64 * kWaves2), 0, st,
+                           static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(kc),
+                           static_cast<const _Float16 *>(vc), static_cast<_Float16 *>(ctx),
+                           static_cast<const _Float16 *>(alibi), pad, H, S, T_cap, scale);
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
 template <int DH>
 int launch(const void *q, const void *kc, const void *vc, void *ctx, const void *alibi, const int64_t *pad, int B,
            int H, int S, int T_cap, hipStream_t st)
@@ -327,6 +643,12 @@ extern "C" int eet_prefill_attention(const void *q, const void *k_cache, const v
         case 32: return launch<32>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
         case 64: return launch<64>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
         case 96: return launch<96>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
-        default: return launch<128>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
+        default: break;
     }
+    // head size 128: the DMA kernel; it addresses a (b, h) cache range with 32-bit byte offsets and reads the
+    // bias row in 4-byte units
+    const bool alibi_ok = alibi == nullptr || (S % 2 == 0 && reinterpret_cast<uintptr_t>(alibi) % 4 == 0);
+    if ((long long)S * 256 < (1ll << 31) && alibi_ok && eet::tuning().prefill_legacy == 0)
+        return launch_dh128(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
+    return launch<128>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);
 }

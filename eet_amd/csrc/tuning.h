@@ -17,6 +17,8 @@ struct Tuning {
     int large_m_tm = 0, large_m_tn = 0, large_m_ksplit = 0;  // ksplit 0: not given
     // EET_MMHA_NSPLIT, EET_MMHA_THREADS, EET_MMHA_UNROLL (0: not given)
     int mmha_nsplit = 0, mmha_threads = 0, mmha_ring = 0;
+    // EET_PREFILL_LEGACY = 1: head size 128 takes the register-staged prefill attention kernel
+    int prefill_legacy = 0;
 };
 
 const Tuning &tuning();

@@ -68,7 +68,10 @@ def test_swiglu_and_residual(gpu):
                                                        (1, 1, 1, 128, False, False), (2, 2, 64, 128, False, False),
                                                        (2, 3, 300, 128, True, False), (1, 2, 257, 64, True, True),
                                                        (1, 2, 1024, 128, False, False), (1, 1, 2500, 128, False, True),
-                                                       (2, 3, 200, 96, True, False), (1, 2, 77, 96, False, True)])
+                                                       (2, 3, 200, 96, True, False), (1, 2, 77, 96, False, True),
+                                                       (2, 2, 600, 128, True, True), (1, 3, 515, 128, False, True),
+                                                       (1, 2, 256, 128, False, False), (2, 1, 255, 128, True, False),
+                                                       (1, 2, 769, 128, False, False)])
 def test_prefill_attention(gpu, B, H, S, dh, use_pad, use_alibi):
     g = torch.Generator().manual_seed(S)
     cap = S + 5
@@ -87,6 +90,14 @@ def test_prefill_attention(gpu, B, H, S, dh, use_pad, use_alibi):
                                       ctx.data_ptr(), row.data_ptr() if use_alibi else None,
                                       padd.data_ptr() if use_pad else None, B, H, S, dh, cap, stream()))
     assert_close(ctx.cpu().numpy(), want, what="prefill ctx")
+
+
+@pytest.mark.parametrize("S,use_alibi", [(300, False), (130, True)])
+def test_prefill_attention_register_staged_kernel_dh128(gpu, tuning, S, use_alibi):
+    """Head size 128 normally takes the DMA kernel; the register-staged one (the path of the other head
+    sizes, and of bias rows the DMA kernel cannot address) is selected here and held to the same oracle."""
+    tuning("EET_PREFILL_LEGACY", 1)
+    test_prefill_attention(gpu, 2, 3, S, 128, True, use_alibi)
 
 
 @pytest.mark.parametrize("B,H,dh,rows,cap", [(4, 3, 64, 9, 16), (8, 32, 128, 100, 128), (3, 2, 32, 0, 8),

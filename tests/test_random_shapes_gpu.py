@@ -96,3 +96,39 @@ def test_attention_random(gpu, B, H, dh, step, cap, use_pad, use_alibi, seed):
                alibi.to(gpu) if use_alibi else None)
     assert_close(ctx.cpu().numpy(), want, what=f"B={B} H={H} dh={dh} step={step} pad={use_pad} alibi={use_alibi}")
     assert np.array_equal(kcd.cpu().numpy(), kcn) and np.array_equal(vcd.cpu().numpy(), vcn)
+
+
+def _prefill_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(n):
+        dh = [128, 128, 64, 128, 96, 128, 32, 128][i % 8]          # mostly the DMA kernel (head size 128)
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 5))
+        S = int(rng.integers(1, [70, 300, 600, 1100][i % 4]))
+        cases.append((B, H, dh, S, S + int(rng.integers(0, 9)), bool(rng.integers(0, 2)), bool(rng.integers(0, 2)),
+                      int(rng.integers(1 << 30))))
+    return cases
+
+
+@pytest.mark.parametrize("B,H,dh,S,cap,use_pad,use_alibi,seed", _prefill_cases(24, 99))
+def test_prefill_attention_random(gpu, B, H, dh, S, cap, use_pad, use_alibi, seed):
+    """Causal prompt attention over random batch / head / length / padding / ALiBi combinations (odd lengths,
+    lengths around the 64-key chunk and 256-query block edges, a padding that covers a whole prompt)."""
+    from eet_amd._lib import check, lib
+    from gpu_util import stream
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = [torch.randn(B, H, S, dh, generator=g).half() for _ in range(3)]
+    kc = torch.randn(B, H, cap, dh, generator=g).half()          # rows past S hold junk that must not be read
+    vc = torch.randn(B, H, cap, dh, generator=g).half()
+    kc[:, :, :S], vc[:, :, :S] = k, v
+    pad = torch.randint(0, S + 1, (B,), generator=g) if use_pad else None
+    want = O.prefill_attention(q.numpy(), k.numpy(), v.numpy(), pad.numpy() if use_pad else None,
+                               O.alibi_mask(H, S) if use_alibi else None)
+    ctx = torch.full((B, S, H * dh), float("nan"), dtype=torch.float16, device=gpu)
+    row = torch.from_numpy(O.alibi_bias(H, S)).to(gpu) if use_alibi else None
+    padd = pad.to(gpu) if use_pad else None
+    qd, kcd, vcd = q.to(gpu), kc.to(gpu), vc.to(gpu)
+    check(lib().eet_prefill_attention(qd.data_ptr(), kcd.data_ptr(), vcd.data_ptr(), ctx.data_ptr(),
+                                      row.data_ptr() if use_alibi else None, padd.data_ptr() if use_pad else None,
+                                      B, H, S, dh, cap, stream()))
+    assert_close(ctx.cpu().numpy(), want, what=f"B={B} H={H} dh={dh} S={S} pad={use_pad} alibi={use_alibi}")

@@ -356,14 +356,16 @@ int launch_small_m(const GemmArgs &a)
     return EET_OK;
 }
 
-// LDS and register budget of an instantiation: slabs and reduction buffer within
-// 64 KiB, and the two register batches small enough not to spill.
+// LDS and register budget of an instantiation: the slabs within 64 KiB, the
+// reduction buffer (which takes over the slabs' memory when both together pass
+// 64 KiB) within 144 of the CU's 160 KiB, and the two register batches small
+// enough not to spill.
 constexpr bool small_m_fits(int nt, int rg, int waves, int u)
 {
     const int mt = (rg + 1) / 2;
     const int stage = waves * u * rg * 1024, red = waves * nt * mt * 1024;
     const int batch_vgprs = 2 * u * (nt + rg) * 4 + nt * mt * 4;
-    return stage <= 65536 && red <= 65536 && batch_vgprs <= (waves == 16 ? 96 : 200);
+    return stage <= 65536 && red <= 147456 && batch_vgprs <= (waves == 16 ? 96 : 200);
 }
 
 template <int RG>
@@ -383,7 +385,7 @@ int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a)
         // the launch shapes pick_small_m can return
         EET_CASE_RMS(1, 8, 2) EET_CASE_RMS(1, 16, 2) EET_CASE_RMS(1, 16, 1)
         EET_CASE_RMS(2, 8, 2) EET_CASE_RMS(2, 8, 1) EET_CASE_RMS(3, 8, 1)
-        EET_CASE_RMS(4, 8, 1)
+        EET_CASE_RMS(4, 8, 1) EET_CASE_RMS(6, 8, 1) EET_CASE_RMS(8, 8, 1)
         return eet::fail(EET_ERR_INVALID_ARGUMENT,
                          "eet_gemm_w8a16_fused: no RMSnorm-prologue kernel for nt=%d waves=%d u=%d", cfg.nt,
                          cfg.waves, cfg.u);
@@ -392,6 +394,7 @@ int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a)
     EET_CASE(2, 4, 2) EET_CASE(2, 8, 2) EET_CASE(2, 16, 2) EET_CASE(2, 8, 4) EET_CASE(2, 16, 1) EET_CASE(2, 8, 1)
     EET_CASE(3, 8, 2) EET_CASE(3, 16, 2) EET_CASE(3, 16, 1) EET_CASE(3, 8, 1)
     EET_CASE(4, 4, 2) EET_CASE(4, 8, 2) EET_CASE(4, 8, 1) EET_CASE(4, 16, 1)
+    EET_CASE(6, 8, 1) EET_CASE(8, 8, 1)
 #undef EET_CASE_RMS
 #undef EET_CASE
     return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no small-M kernel for nt=%d waves=%d u=%d (M=%d)",
@@ -406,22 +409,28 @@ int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a)
 // activation traffic (every workgroup reads all M x K activations; they come
 // from L2 at about 0.37 of the cost of an HBM byte, 1 KiB per 8 rows and k-tile
 // against NT KiB of weights), the third a mild preference for several
-// workgroups per CU.  Fitted to sweeps over NT = 1..4 on MI355X at M = 8, 16, 32 on
-// the LLaMA-7B shapes (N/16 = 768, 256, 1376, 256 n-tiles) and the Baichuan-13B
-// shapes (960, 320, 1712, 320), whose order it reproduces.  The SwiGLU epilogue
-// needs an even NT (gate / up pairs).  One n-tile per workgroup runs with 16
-// wavefronts when there are few workgroups (more loads in flight per CU).
+// workgroups per CU.  Fitted to sweeps over NT = 1..4, 6, 8 on MI355X at M = 8, 16, 32
+// on the LLaMA-7B shapes (N/16 = 768, 256, 1376, 256 n-tiles) and the Baichuan-13B
+// shapes (960, 320, 1712, 320), whose order it reproduces: e.g. 1376 n-tiles are 5.4
+// per CU, which both NT = 2 (688 workgroups, three rounds) and NT = 6 (230 workgroups,
+// one round) turn into a load of 6, the latter with a third of the activation reads
+// (M = 32: 20.1 against 28.1 us).  The SwiGLU epilogue needs an even NT (gate / up
+// pairs).  One n-tile per workgroup runs with 16 wavefronts when there are few
+// workgroups (more loads in flight per CU).
 SmallMConfig pick_small_m(int M, int N, int K, int epi, bool rms)
 {
     const int ntiles = N / 16;
     (void)K;
     int best_nt = 0;
     double best = 0.0;
-    for (int nt = (epi == kEpiSwiglu) ? 2 : 1; nt <= 4; nt += (epi == kEpiSwiglu) ? 2 : 1) {
+    for (int nt : {1, 2, 3, 4, 6, 8}) {
+        if (epi == kEpiSwiglu && nt % 2 != 0)
+            continue;
         const int wgs = (ntiles + nt - 1) / nt;
         const double load = (double)((wgs + 255) / 256) * nt;
         const double per_cu = wgs / 256.0 < 4.0 ? wgs / 256.0 : 4.0;
-        const double cost = load * (1.0 + 0.37 * M / (8.0 * nt)) * (1.0 + 0.1 / per_cu);
+        // NT = 6 and 8 leave one workgroup per CU: taken only where they win by more than 3 %
+        const double cost = load * (1.0 + 0.37 * M / (8.0 * nt)) * (1.0 + 0.1 / per_cu) * (nt > 4 ? 1.03 : 1.0);
         if (best_nt == 0 || cost < best) {
             best = cost;
             best_nt = nt;

@@ -96,6 +96,44 @@ def test_large_m_path(gpu):
         assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32), what=f"M={M}")
 
 
+SMALL_M_SHAPES = ["1,8,2", "1,16,2", "1,16,1", "2,8,2", "2,8,1", "3,8,1", "4,8,1", "6,8,1", "8,8,1"]   # NT, wavefronts, k-tiles per batch
+
+
+@pytest.mark.parametrize("cfg", SMALL_M_SHAPES)
+def test_small_m_launch_shapes(gpu, tuning, cfg):
+    """Every launch shape the small-M dispatcher can pick (selected with the tuning override), for the
+    three row-group counts (M <= 8, <= 16, <= 32), on channel counts that leave the last workgroup
+    ragged and k ranges that leave the wavefronts uneven shares: plain, RMSnorm prologue + residual,
+    RMSnorm prologue + SwiGLU (an odd NT cannot pair gate / up tiles: the dispatcher's own choice runs)."""
+    from eet_amd.ops import interleave_gate_up
+    tuning("EET_GEMM_SMALL_M_CONFIG", cfg)
+    eps = 1e-6
+    for (M, K, N) in [(5, 576, 208), (16, 2752, 1104), (27, 704, 400)]:
+        x, u, p, s = make(M, K, N, M + K + N)
+        g = torch.Generator().manual_seed(M)
+        gamma = (1 + 0.1 * torch.randn(K, generator=g)).half()
+        res = torch.randn(M, N, generator=g).half()
+        xd, pd, sd = x.to(gpu), p.to(gpu), s.to(gpu)
+        ref = O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32)
+        assert_close(gemm(xd, pd, sd, M, N, K).cpu().numpy(), ref, what=f"{cfg} plain M={M}")
+        x32 = x.numpy().astype(np.float32)
+        xn = x32 / np.sqrt((x32 * x32).mean(-1, keepdims=True) + np.float32(eps)) * gamma.numpy().astype(np.float32)
+        deq = u.numpy().astype(np.float32) * s.numpy().astype(np.float32)[None, :]
+        got = fused(xd, pd, sd, M, N, K, 1, res.to(gpu), gamma.to(gpu), eps).cpu().numpy()
+        assert_close(got, O.residual_add((xn @ deq).astype(np.float16), res.numpy()), rtol=1e-2, atol=3e-3,
+                     what=f"{cfg} rms+residual M={M}")
+        F = N // 2 + 8
+        wg = (torch.randn(K, F, generator=g) * 0.02).half()
+        wu = (torch.randn(K, F, generator=g) * 0.02).half()
+        ug, pg, sg = eet_amd.quant_weights(wg, torch.int8, True)
+        uu, pu, su = eet_amd.quant_weights(wu, torch.int8, True)
+        w01, s01 = interleave_gate_up(pg, sg, pu, su)
+        got = fused(xd, w01.to(gpu), s01.to(gpu), M, 2 * F, K, 2, None, gamma.to(gpu), eps).cpu().numpy()
+        gate = xn @ (ug.numpy().astype(np.float32) * sg.numpy().astype(np.float32)[None, :])
+        up = xn @ (uu.numpy().astype(np.float32) * su.numpy().astype(np.float32)[None, :])
+        assert_close(got, up * gate / (1 + np.exp(-gate)), rtol=1e-2, atol=3e-3, what=f"{cfg} rms+swiglu M={M}")
+
+
 LARGE_M_TILES = ["8,4", "4,5", "4,4", "4,2", "2,2"]   # m-tiles, n-tiles per wavefront
 
 

@@ -66,9 +66,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 4, j = lane & 15;
-    const int bh = blockIdx.y, b = bh / H, h = bh % H;
+    // all (batch, head) pairs of the last (longest) query block are handed out first, then the one before, ...
+    const int bh = blockIdx.x, b = bh / H, h = bh % H;
     const int q_blocks = (S + kBQ - 1) / kBQ;
-    const int q0 = (q_blocks - 1 - (int)blockIdx.x) * kBQ;  // late (long) query blocks first
+    const int q0 = (q_blocks - 1 - (int)blockIdx.y) * kBQ;
     const int padb = pad ? (int)min((int64_t)S, max((int64_t)0, pad[b])) : 0;
 
     const _Float16 *kbase = k_cache + (size_t)bh * T_cap * DH;
@@ -341,9 +342,12 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 4, j = lane & 15;
-    const int bh = blockIdx.y, b = bh / H, h = bh % H;
+    // Workgroups are handed out in index order: all (batch, head) pairs of the last query block first, then
+    // those of the one before, so the long blocks start first over the whole launch and the short ones fill
+    // the tail (with the block index running fastest the last CU to finish held up to a fifth of the launch).
+    const int bh = blockIdx.x, b = bh / H, h = bh % H;
     const int q_blocks = (S + kBQ2 - 1) / kBQ2;
-    const int q0 = (q_blocks - 1 - (int)blockIdx.x) * kBQ2;  // late (long) query blocks first
+    const int q0 = (q_blocks - 1 - (int)blockIdx.y) * kBQ2;
     const int padb = pad ? (int)min((int64_t)S, max((int64_t)0, pad[b])) : 0;
 
     const _Float16 *kbase = k_cache + (size_t)bh * T_cap * kD;
@@ -598,7 +602,7 @@ int launch_dh128(const void *q, const void *kc, const void *vc, void *ctx, const
                  int H, int S, int T_cap, hipStream_t st)
 {
     const float scale = (float)(_Float16)(1.0f / sqrtf(128.0f));
-    dim3 grid((S + kBQ2 - 1) / kBQ2, B * H);
+    dim3 grid(B * H, (S + kBQ2 - 1) / kBQ2);
     if (alibi != nullptr)
         hipLaunchKernelGGL((prefill_attention_dh128_kernel<true>), grid, dim3(64 * kWaves2), 0, st,
                            static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(kc),
@@ -618,7 +622,7 @@ int launch(const void *q, const void *kc, const void *vc, void *ctx, const void 
            int H, int S, int T_cap, hipStream_t st)
 {
     const float scale = (float)(_Float16)(1.0f / sqrtf((float)DH));
-    dim3 grid((S + kBQ - 1) / kBQ, B * H);
+    dim3 grid(B * H, (S + kBQ - 1) / kBQ);
     hipLaunchKernelGGL((prefill_attention_kernel<DH>), grid, dim3(kThreads), 0, st, static_cast<const _Float16 *>(q),
                        static_cast<const _Float16 *>(kc), static_cast<const _Float16 *>(vc),
                        static_cast<_Float16 *>(ctx), static_cast<const _Float16 *>(alibi), pad, H, S, T_cap, scale);
@@ -637,7 +641,9 @@ extern "C" int eet_prefill_attention(const void *q, const void *k_cache, const v
                 "eet_prefill_attention: bad sizes B=%d H=%d S=%d T_cap=%d", B, H, S, T_cap);
     EET_REQUIRE(dh == 32 || dh == 64 || dh == 96 || dh == 128, EET_ERR_UNSUPPORTED_SHAPE,
                 "eet_prefill_attention: head size %d not supported (32, 64, 96, 128)", dh);
-    EET_REQUIRE((long long)B * H <= 65535, EET_ERR_UNSUPPORTED_SHAPE, "eet_prefill_attention: B*H too large");
+    // grid: (batch, head) pairs in x, query blocks in y
+    EET_REQUIRE((long long)B * H < (1ll << 31) && (S + kBQ - 1) / kBQ <= 65535, EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_prefill_attention: B*H = %lld or S = %d too large", (long long)B * H, S);
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (dh) {
         case 32: return launch<32>(q, k_cache, v_cache, ctx, alibi, pad, B, H, S, T_cap, st);

@@ -604,7 +604,7 @@ def main():
     gbs = step_bytes / sec / 1e9
     per_launch_us = sec / launches * 1e6
     # the same chain of launches as pure reads of the same weight buffers: what the machine allows
-    # (with the GEMM's own grids, and with two and four times as many workgroups: the best of the three counts)
+    # (256 workgroups per launch, 688 for gate|up, and two and four times as many: the best of the three counts)
     probe_sec = min(time_gemm_pass(torch, L, fused, acts, outs, M, max(3, args.steps // 2), 1, probe=True,
                                    probe_grid_scale=sc)[0] for sc in (1, 2, 4))
     weight_bytes = sum(w.numel() for layer in fused for (w, _, _) in layer.values())
@@ -631,7 +631,8 @@ def main():
                      "stream_ceiling": {"GB/s": round(ceiling_gbs, 1), "frac_of_peak": round(ceiling_gbs / HBM_PEAK_GBS, 4),
                                         "ms_per_step": round(probe_sec * 1e3, 4),
                                         "what": "the same 128 launches per step as read-only streams of the same weight "
-                                                "buffers (eet_hbm_stream_probe, same grids): the rate this machine "
+                                                "buffers (eet_hbm_stream_probe; 256 workgroups per launch, 688 for gate|up, also at "
+                                                "twice and four times as many, best of the three): the rate this machine "
                                                 "allows a chain of dependent launches of these sizes"},
                      "frac_of_stream_ceiling": round(step_bytes / sec / (weight_bytes / probe_sec), 4)},
         "host_wall_ms_per_step": round(wall * 1e3, 4),

@@ -329,6 +329,24 @@ __device__ __forceinline__ int row_swz(int r) { return ((r & 7) << 1) | ((r >> 3
 
 typedef short short4v __attribute__((ext_vector_type(4)));
 
+// Maximum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 with the lane-swap instructions of gfx950 (two vector
+// instructions per step, no trip through the LDS crossbar as a bpermute takes).  v_permlane16_swap exchanges the
+// odd 16-lane rows of its first operand with the even rows of its second: on two copies of v it leaves (even rows
+// duplicated, odd rows duplicated); v_permlane32_swap does the same with the two 32-lane halves.  Written as
+// assembly because the compiler builtin dropped the second result; the s_nop's cover the wait states the
+// instruction needs after a vector write of its operands and before a vector read of its results.
+__device__ __forceinline__ float max_over_lane_groups(float v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    float x = v, y = v;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
+    x = y = fmaxf(x, y);
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
+    v = fmaxf(x, y);
+#endif
+    return v;
+}
+
 template <bool ALIBI>
 __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attention_dh128_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_cache, const _Float16 *__restrict__ v_cache,
@@ -461,22 +479,29 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
             // Without a bias the scale is applied inside the exponent's argument (one fused multiply-add per
             // element instead of a multiply and a subtract): the maximum is taken over the raw products and
             // scaled once (the scale is positive).
+            if (ALIBI) {
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        sacc[qt][kt][r] = sacc[qt][kt][r] * scale2 + (float)bias4[kt][r] * kLog2e;
+            }
+            // one branch around all sixteen tests (inside the loop below it became a branch per score)
+            if (need_mask) {
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int key = kc0 + 16 * kt + 4 * g + r;
+                        sacc[qt][kt][r] = (key > qi || key < padb) ? -INFINITY : sacc[qt][kt][r];
+                    }
+            }
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float s = sacc[qt][kt][r];
-                    if (ALIBI)
-                        s = s * scale2 + (float)bias4[kt][r] * kLog2e;
-                    if (need_mask) {
-                        const int key = kc0 + 16 * kt + 4 * g + r;
-                        s = (key > qi || key < padb) ? -INFINITY : s;
-                    }
-                    sacc[qt][kt][r] = s;
-                    cmax = fmaxf(cmax, s);
-                }
-            cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
-            cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+                for (int r = 0; r < 4; ++r)
+                    cmax = fmaxf(cmax, sacc[qt][kt][r]);
+            cmax = max_over_lane_groups(cmax);
             if (!ALIBI)
                 cmax *= scale2;
             const float m_new = fmaxf(m_run[qt], cmax);

@@ -92,6 +92,29 @@ def test_prefill_attention(gpu, B, H, S, dh, use_pad, use_alibi):
     assert_close(ctx.cpu().numpy(), want, what="prefill ctx")
 
 
+@pytest.mark.parametrize("dh", [128, 64])
+@pytest.mark.parametrize("dominant", [1, 6, 11, 12, 37, 62])
+def test_prefill_attention_one_dominant_key(gpu, dh, dominant):
+    """One key whose score towers over the rest (q . k / sqrt(dh) ~ +40 against O(1)), at every position class
+    of the 64-key chunk layout: the running maximum has to be taken over all keys of a chunk, or the weight of
+    that key overflows fp16 (e^40) and the row comes out as NaN.  Every later query then returns that key's V row."""
+    B, H, S = 1, 2, 192
+    g = torch.Generator().manual_seed(dominant)
+    q = torch.full((B, H, S, dh), 2.0).half()
+    k = (torch.randn(B, H, S, dh, generator=g) * 0.05).half()
+    v = torch.randn(B, H, S, dh, generator=g).half()
+    for pos in (dominant, 64 + dominant):
+        k[:, :, pos] = 40.0 * (dh ** 0.5) / (2.0 * dh)
+    want = O.prefill_attention(q.numpy(), k.numpy(), v.numpy(), None, None)
+    ctx = torch.empty(B, S, H * dh, dtype=torch.float16, device=gpu)
+    qd, kd, vd = q.to(gpu), k.to(gpu), v.to(gpu)
+    check(lib().eet_prefill_attention(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), ctx.data_ptr(), None, None,
+                                      B, H, S, dh, S, stream()))
+    got = ctx.cpu().numpy()
+    assert np.isfinite(got).all()
+    assert_close(got, want, what=f"dominant key {dominant}")
+
+
 @pytest.mark.parametrize("S,use_alibi", [(300, False), (130, True)])
 def test_prefill_attention_register_staged_kernel_dh128(gpu, tuning, S, use_alibi):
     """Head size 128 normally takes the DMA kernel; the register-staged one (the path of the other head

@@ -49,6 +49,24 @@ constexpr int kQT = 2;     // 16-query tiles per wavefront
 
 __device__ __forceinline__ int vt_swizzle(int d) { return (d & 15) ^ ((d >> 3) & 15); }
 
+// Maximum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 with the lane-swap instructions of gfx950 (two vector
+// instructions per step, no trip through the LDS crossbar as a bpermute takes).  v_permlane16_swap exchanges the
+// odd 16-lane rows of its first operand with the even rows of its second: on two copies of v it leaves (even rows
+// duplicated, odd rows duplicated); v_permlane32_swap does the same with the two 32-lane halves.  Written as
+// assembly because the compiler builtin dropped the second result; the s_nop's cover the wait states the
+// instruction needs after a vector write of its operands and before a vector read of its results.
+__device__ __forceinline__ float max_over_lane_groups(float v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    float x = v, y = v;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
+    x = y = fmaxf(x, y);
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
+    v = fmaxf(x, y);
+#endif
+    return v;
+}
+
 template <int DH>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void prefill_attention_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_cache, const _Float16 *__restrict__ v_cache,
@@ -218,17 +236,24 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float s = sacc[qt][kt][r] * scale2 + (float)bias4[kt][r] * kLog2e;
-                    if (need_mask) {
+                for (int r = 0; r < 4; ++r)
+                    sacc[qt][kt][r] = sacc[qt][kt][r] * scale2 + (float)bias4[kt][r] * kLog2e;
+            // one branch around all sixteen tests (inside the loop above it becomes a branch per score)
+            if (need_mask) {
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
                         const int key = kc0 + 16 * kt + 4 * g + r;
-                        s = (key > qi || key < padb) ? -INFINITY : s;
+                        sacc[qt][kt][r] = (key > qi || key < padb) ? -INFINITY : sacc[qt][kt][r];
                     }
-                    sacc[qt][kt][r] = s;
-                    cmax = fmaxf(cmax, s);
-                }
-            cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
-            cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+            }
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    cmax = fmaxf(cmax, sacc[qt][kt][r]);
+            cmax = max_over_lane_groups(cmax);
             const float m_new = fmaxf(m_run[qt], cmax);
             const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
             const float corr = __builtin_amdgcn_exp2f(m_run[qt] - m_safe);  // 0 while nothing has been seen
@@ -243,9 +268,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
                 }
             l_run[qt] = l_run[qt] * corr + psum;  // per-lane share; lanes of a query are summed at the end
             m_run[qt] = m_new;
+            // the accumulator is rescaled only when some query's maximum moved (rare after the first chunks)
+            if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                oacc[qt][dt] *= corr;
+                for (int dt = 0; dt < DT; ++dt)
+                    oacc[qt][dt] *= corr;
+            }
             // P^T operands: contraction slots of lane group g = keys 4g..4g+3 of tile 2*hf, then of tile 2*hf+1
 #pragma unroll
             for (int hf = 0; hf < 2; ++hf) {
@@ -328,24 +356,6 @@ __device__ __forceinline__ int k_swz(int r) { return r & 15; }
 __device__ __forceinline__ int row_swz(int r) { return ((r & 7) << 1) | ((r >> 3) & 1); }
 
 typedef short short4v __attribute__((ext_vector_type(4)));
-
-// Maximum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 with the lane-swap instructions of gfx950 (two vector
-// instructions per step, no trip through the LDS crossbar as a bpermute takes).  v_permlane16_swap exchanges the
-// odd 16-lane rows of its first operand with the even rows of its second: on two copies of v it leaves (even rows
-// duplicated, odd rows duplicated); v_permlane32_swap does the same with the two 32-lane halves.  Written as
-// assembly because the compiler builtin dropped the second result; the s_nop's cover the wait states the
-// instruction needs after a vector write of its operands and before a vector read of its results.
-__device__ __forceinline__ float max_over_lane_groups(float v)
-{
-#if defined(__HIP_DEVICE_COMPILE__)
-    float x = v, y = v;
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
-    x = y = fmaxf(x, y);
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
-    v = fmaxf(x, y);
-#endif
-    return v;
-}
 
 template <bool ALIBI>
 __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attention_dh128_kernel(

@@ -26,12 +26,15 @@
 // numbered so that the ones sharing a weight column block run on the same XCD
 // (workgroup i lands on XCD i % 8) and hit its L2.
 //
-// A stage holds TM m-tiles of 2 KiB: [row half b][row r (8)][position (8)] x
-// 16 B, where position p of row (b, r) holds piece p ^ ((r >> 1) | (b << 2)) of
-// the row's eight 16-byte pieces.  One DMA instruction fills 1 KiB (8 rows x
-// 128 B, whole cache lines; the XOR only permutes lanes within a line), and the
-// MFMA operand read of lane (g, j) -- piece 2g+h of row j -- hits 16 distinct
-// 16-byte bank groups per 16 lanes.
+// A stage holds TM / 2 blocks of 4 KiB, one per pair of m-tiles (2u, 2u + 1):
+// 16 "super-rows" of 256 B, super-row j holding row j of both m-tiles.  The MFMA
+// operand of lane (g, j) for m-tile 2u + e, k half h -- the 16-byte piece 2g + h
+// of row j -- sits at slot (4 * (2e + h) + g) ^ j of super-row j.  With that
+// placement a ds_read_b128 of the whole wavefront runs at the full 256 B/clk of
+// the LDS (measured: 128-byte rows with any XOR of the row index reach 150 B/clk).
+// One DMA instruction fills 1 KiB = four super-rows; its lanes fetch whole
+// 128-byte lines of eight activation rows (the XOR only permutes the lanes
+// within a line).
 #include "gemm_common.h"
 #include "tuning.h"
 
@@ -54,6 +57,7 @@ struct DmaShape {
     static constexpr int kRowGroups = TM * 2;           // DMA instructions per k-tile (8 rows each)
     static constexpr int kPerWave = kRowGroups / WNW;   // ... per wavefront
     static_assert(kRowGroups % WNW == 0, "row groups must divide over the wavefronts");
+    static_assert(TM % 2 == 0, "a stage block holds a pair of m-tiles");
     static_assert(kDmaStages * kStageVec * 16 <= 65536, "the stage ring must fit 64 KiB");
 };
 
@@ -106,17 +110,20 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
     for (int t = 0; t < TN; ++t)
         wtile[t] = (unsigned)min(nt0 + t, ntiles - 1) * (unsigned)ktiles * 1024u;
 
-    // DMA source of this lane for row group rg = wave * kPerWave + i: row
-    // 8*rg + lane/8, piece (lane%8) ^ swizzle.
+    // DMA instruction rg = wave * kPerWave + i fills slots [64 rg, 64 rg + 64): block u = rg / 4,
+    // super-rows 4 (rg % 4) .. + 3.  Lane l writes slot s = l % 16 of super-row sj = 4 (rg % 4) + l / 16,
+    // which holds piece 2 pg + h of row sj of m-tile 2u + e, where 4 (2e + h) + pg = s ^ sj.
     int aoff[S::kPerWave];
 #pragma unroll
     for (int i = 0; i < S::kPerWave; ++i) {
-        const int rg = wave * S::kPerWave + i, r = lane >> 3, b = rg & 1;
-        const int piece = (lane & 7) ^ ((r >> 1) | (b << 2));
-        aoff[i] = (8 * rg + r) * K * 2 + piece * 16;
+        const int rg = wave * S::kPerWave + i, u = rg >> 2, sj = 4 * (rg & 3) + (lane >> 4);
+        const int p = (lane & 15) ^ sj, pg = p & 3, h = (p >> 2) & 1, e = p >> 3;
+        aoff[i] = ((2 * u + e) * 16 + sj) * K * 2 + (2 * pg + h) * 16;
     }
-    const int swz = ((j & 7) >> 1) | ((j >> 3) << 2);
-    const int rs0 = (j >> 3) * 64 + (j & 7) * 8 + ((2 * g) ^ swz), rs1 = rs0 ^ 1;
+    int rs[4];  // operand slot of this lane within a block, by 2e + h
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+        rs[c] = j * 16 + ((4 * c + g) ^ j);
 
     floatx4 acc[TN][TM];
 #pragma unroll
@@ -154,14 +161,14 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
         __builtin_amdgcn_sched_barrier(0);
         load_w(wb, kbeg + min(kt + 2, nk - 1));
         half8 aop[2][2];
-        aop[0][0] = __builtin_bit_cast(half8, cur[rs0]);
-        aop[0][1] = __builtin_bit_cast(half8, cur[rs1]);
+        aop[0][0] = __builtin_bit_cast(half8, cur[rs[0]]);
+        aop[0][1] = __builtin_bit_cast(half8, cur[rs[1]]);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int mt = 0; mt < TM; ++mt) {
             if (mt + 1 < TM) {
-                aop[(mt + 1) & 1][0] = __builtin_bit_cast(half8, cur[(mt + 1) * 128 + rs0]);
-                aop[(mt + 1) & 1][1] = __builtin_bit_cast(half8, cur[(mt + 1) * 128 + rs1]);
+                aop[(mt + 1) & 1][0] = __builtin_bit_cast(half8, cur[((mt + 1) >> 1) * 256 + rs[2 * ((mt + 1) & 1)]]);
+                aop[(mt + 1) & 1][1] = __builtin_bit_cast(half8, cur[((mt + 1) >> 1) * 256 + rs[2 * ((mt + 1) & 1) + 1]]);
             }
 #pragma unroll
             for (int t = 0; t < TN; ++t) {

@@ -7,7 +7,7 @@
 // A workgroup of WNW wavefronts side by side owns a block tile of TM*16 rows x
 // WNW*TN*16 channels; each wavefront owns TM x TN tiles of
 // v_mfma_f32_16x16x32_f16 (TM*TN*4 fp32 accumulator registers).  What bounds
-// such a kernel on a CU is the LDS port (128 B/clk) against the matrix cores
+// such a kernel on a CU is the LDS port (256 B/clk at best) against the matrix cores
 // (4 x 1024 flop/clk): a wavefront tile of WM x WN outputs needs (WM + WN) * 2 B
 // of operands per k for 2 * WM * WN flop, so wavefront tiles are made large
 // (128 x 64 where M allows) and only one operand goes through LDS:

@@ -648,7 +648,7 @@ def main():
 
     if not args.no_sweep:
         sweep = {}
-        for m in (1, 4, 8, 16, 32):
+        for m in (1, 2, 4, 8, 16, 32):
             s, _, n = time_gemm_pass(torch, L, fused, acts, outs, m, max(3, args.steps // 4), 1)
             b = pass_bytes(fused, m)
             sweep[f"M={m}"] = {"GB/s": round(b / s / 1e9, 1), "pct_peak": round(100 * b / s / 1e9 / HBM_PEAK_GBS, 2)}

@@ -400,11 +400,18 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
             qop[qt][c] = *reinterpret_cast<const half8 *>(qbase + (size_t)qi * kD + 32 * c + 8 * g);
     }
     floatx4 oacc[2][DT];
-    float m_run[2], l_run[2];
+    // The softmax denominators ride along as one more accumulator tile per query tile: P^T times a V^T operand of
+    // ones leaves, in every row, the sum over the keys of the weights as the matrix cores see them (rounded to
+    // fp16, like the numerator) -- two matrix instructions per chunk and tile instead of sixteen vector adds per
+    // lane, and no cross-lane sum at the end.
+    floatx4 lacc[2];
+    float m_run[2];
+    const half8 ones8 = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f,
+                         (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
         m_run[qt] = -INFINITY;
-        l_run[qt] = 0.f;
+        lacc[qt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
             oacc[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -517,23 +524,20 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
             const float m_new = fmaxf(m_run[qt], cmax);
             const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
             const float corr = __builtin_amdgcn_exp2f(m_run[qt] - m_safe);  // 0 while nothing has been seen
-            float psum = 0.f;
             float p[4][4];
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
+                for (int r = 0; r < 4; ++r)
                     p[kt][r] = ALIBI ? __builtin_amdgcn_exp2f(sacc[qt][kt][r] - m_safe)
                                      : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qt][kt][r], scale2, -m_safe));
-                    psum += p[kt][r];
-                }
-            l_run[qt] = l_run[qt] * corr + psum;
             m_run[qt] = m_new;
-            // the accumulator is rescaled only when some query's maximum moved (rare after the first chunks)
+            // the accumulators are rescaled only when some query's maximum moved (rare after the first chunks)
             if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
                     oacc[qt][dt] *= corr;
+                lacc[qt] *= corr;
             }
 #pragma unroll
             for (int hf = 0; hf < 2; ++hf) {
@@ -571,6 +575,12 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
                         oacc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop, pop[qt][hf], oacc[qt][dt], 0, 0, 0);
             }
         }
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt)
+                if (MASK & (1 << qt))
+                    lacc[qt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones8, pop[qt][hf], lacc[qt], 0, 0, 0);
         // the transposing reads (two per operand) two operands ahead of the matrix instructions
         {
             constexpr int kPer = (MASK == 3) ? 2 : 1;
@@ -580,7 +590,7 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
                 __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             }
-            __builtin_amdgcn_sched_group_barrier(0x008, 2 * kPer, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 4 * kPer, 0);
         }
     };
 
@@ -613,9 +623,7 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
 
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
-        float l = l_run[qt];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
+        const float l = lacc[qt][0];   // every row of the tile holds the sum for query j
         const int qi = tq0[qt] + j;
         if (qi >= S)
             continue;

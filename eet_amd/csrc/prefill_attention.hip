@@ -345,7 +345,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 // ds_read_b64_tr_b16, which hands lane i column i of a 4 x 16 block of halves.
 // ---------------------------------------------------------------------------
 constexpr int kD = 128;
-constexpr int kWaves2 = 8, kBQ2 = 256, kStages = 4;
+constexpr int kBQ2 = 256, kStages = 4;
 constexpr int kStageVec = 2 * 1024 + 16;   // u32x4 per stage: K rows, V rows, bias row (+ padding)
 
 // Measured on MI355X with 8 wavefronts reading back to back: a 16-byte operand read (lane = row) runs at
@@ -357,8 +357,12 @@ __device__ __forceinline__ int row_swz(int r) { return ((r & 7) << 1) | ((r >> 3
 
 typedef short short4v __attribute__((ext_vector_type(4)));
 
-template <bool ALIBI>
-__global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attention_dh128_kernel(
+// NQT 16-query tiles per wavefront, WAVES wavefronts: 256 queries per workgroup either way.  <2, 8>: two wavefronts
+// per SIMD with 256 registers each, every K and V operand read feeds two tiles; <1, 16>: four wavefronts per SIMD,
+// twice the operand reads (the LDS has the room), faster on short prompts, where a workgroup sees few chunks and
+// its start-up and the diagonal chunks weigh more.
+template <bool ALIBI, int NQT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4))) void prefill_attention_dh128_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_cache, const _Float16 *__restrict__ v_cache,
     _Float16 *__restrict__ ctx, const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, int H, int S,
     int T_cap, float scale)
@@ -389,27 +393,32 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
     const __amdgpu_buffer_rsrc_t ars = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<_Float16 *>(ALIBI ? alibi + (size_t)h * S : q), 0, ALIBI ? (unsigned)S * 2u : 0u, 0x00020000);
 
-    // the two query tiles of this wavefront
-    int tq0[2] = {q0 + 16 * wave, q0 + 16 * (wave + kWaves2)};
-    half8 qop[2][DC];
+    static_assert(NQT * WAVES == 16 && (NQT == 1 || NQT == 2), "256 queries per workgroup");
+    constexpr int KI = 16 / WAVES;   // DMA instructions per wavefront for the K rows of a chunk (and for the V rows)
+    // the query tiles of this wavefront: one early, one late (the causal triangle is split evenly)
+    int tq0[NQT];
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
+    for (int qt = 0; qt < NQT; ++qt)
+        tq0[qt] = q0 + 16 * (wave + qt * WAVES);
+    half8 qop[NQT][DC];
+#pragma unroll
+    for (int qt = 0; qt < NQT; ++qt) {
         const int qi = min(tq0[qt] + j, S - 1);
 #pragma unroll
         for (int c = 0; c < DC; ++c)
             qop[qt][c] = *reinterpret_cast<const half8 *>(qbase + (size_t)qi * kD + 32 * c + 8 * g);
     }
-    floatx4 oacc[2][DT];
+    floatx4 oacc[NQT][DT];
     // The softmax denominators ride along as one more accumulator tile per query tile: P^T times a V^T operand of
     // ones leaves, in every row, the sum over the keys of the weights as the matrix cores see them (rounded to
     // fp16, like the numerator) -- two matrix instructions per chunk and tile instead of sixteen vector adds per
     // lane, and no cross-lane sum at the end.
-    floatx4 lacc[2];
-    float m_run[2];
+    floatx4 lacc[NQT];
+    float m_run[NQT];
     const half8 ones8 = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f,
                          (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
+    for (int qt = 0; qt < NQT; ++qt) {
         m_run[qt] = -INFINITY;
         lacc[qt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -418,11 +427,11 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
     }
 
     // DMA: instruction t of a chunk fills rows 4t .. 4t+3 (1 KiB); lane l carries position l % 16 of row
-    // 4t + l / 16, i.e. piece (l % 16) ^ swz(row).  Wavefront w issues instructions 2w and 2w + 1 of K and of V.
-    int dma_off_k[2], dma_off_v[2];   // byte offset of this lane's piece within a chunk, for its two instructions
+    // 4t + l / 16, i.e. piece (l % 16) ^ swz(row).  Wavefront w issues instructions KI w .. KI w + KI - 1 of K and of V.
+    int dma_off_k[KI], dma_off_v[KI];   // byte offset of this lane's piece within a chunk, per instruction
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int row = 4 * (2 * wave + i) + (lane >> 4);
+    for (int i = 0; i < KI; ++i) {
+        const int row = 4 * (KI * wave + i) + (lane >> 4);
         dma_off_k[i] = row * (kD * 2) + (((lane & 15) ^ k_swz(row)) << 4);
         dma_off_v[i] = row * (kD * 2) + (((lane & 15) ^ row_swz(row)) << 4);
     }
@@ -430,9 +439,9 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
         u32x4 *st = lds + stage * kStageVec;
         const int base = kc0 * (kD * 2);   // in the lane offset: the range check of a buffer load covers it
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(krs, st + (2 * wave + i) * 64, 16, base + dma_off_k[i], 0, 0, 0);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(vrs, st + 1024 + (2 * wave + i) * 64, 16, base + dma_off_v[i], 0, 0, 0);
+        for (int i = 0; i < KI; ++i) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(krs, st + (KI * wave + i) * 64, 16, base + dma_off_k[i], 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(vrs, st + 1024 + (KI * wave + i) * 64, 16, base + dma_off_v[i], 0, 0, 0);
         }
         if (ALIBI)   // the chunk's 64 bias terms (128 B): every wavefront writes the same bytes
             __builtin_amdgcn_raw_ptr_buffer_load_lds(ars, st + 2048, 4, kc0 * 2 + (lane & 31) * 4, 0, 0, 0);
@@ -449,9 +458,9 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
         constexpr int MASK = decltype(mask_c)::value;
         const u32x4 *kst = st;
         const unsigned char *vst = reinterpret_cast<const unsigned char *>(st + 1024);
-        floatx4 sacc[2][4];
+        floatx4 sacc[NQT][4];
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt)
+        for (int qt = 0; qt < NQT; ++qt)
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
                 sacc[qt][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -462,14 +471,14 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
             for (int c = 0; c < DC; ++c) {
                 const half8 kop = __builtin_bit_cast(half8, kst[row * 16 + ((4 * c + g) ^ k_swz(row))]);
 #pragma unroll
-                for (int qt = 0; qt < 2; ++qt)
+                for (int qt = 0; qt < NQT; ++qt)
                     if (MASK & (1 << qt))
                         sacc[qt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop, qop[qt][c], sacc[qt][kt], 0, 0, 0);
             }
         }
         // operand reads three ahead of the matrix instructions that use them
         {
-            constexpr int kPer = (MASK == 3) ? 2 : 1;
+            constexpr int kPer = (MASK == 3) ? 2 : 1;   // query tiles taking part
             __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
 #pragma unroll
             for (int n = 0; n < 13; ++n) {
@@ -485,9 +494,9 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
             for (int kt = 0; kt < 4; ++kt)
                 bias4[kt] = *reinterpret_cast<const half4 *>(bst + 16 * kt + 4 * g);
         }
-        half8 pop[2][2];
+        half8 pop[NQT][2];
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
+        for (int qt = 0; qt < NQT; ++qt) {
             if (!(MASK & (1 << qt)))
                 continue;
             const int qi = tq0[qt] + j;
@@ -570,7 +579,7 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
                 const half4 lo = __builtin_bit_cast(half4, part[0]), hi = __builtin_bit_cast(half4, part[1]);
                 const half8 vop = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
-                for (int qt = 0; qt < 2; ++qt)
+                for (int qt = 0; qt < NQT; ++qt)
                     if (MASK & (1 << qt))
                         oacc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop, pop[qt][hf], oacc[qt][dt], 0, 0, 0);
             }
@@ -578,12 +587,12 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
-            for (int qt = 0; qt < 2; ++qt)
+            for (int qt = 0; qt < NQT; ++qt)
                 if (MASK & (1 << qt))
                     lacc[qt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones8, pop[qt][hf], lacc[qt], 0, 0, 0);
         // the transposing reads (two per operand) two operands ahead of the matrix instructions
         {
-            constexpr int kPer = (MASK == 3) ? 2 : 1;
+            constexpr int kPer = (MASK == 3) ? 2 : 1;   // query tiles taking part
             __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
             for (int n = 0; n < 2 * DT - 2; ++n) {
@@ -597,11 +606,12 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
     auto chunk = [&](int c) {
         const int kc0 = k_begin + c * kBK;
         const u32x4 *st = lds + (c % kStages) * kStageVec;
-        const bool t0 = kc0 <= tq0[0] + 15 && tq0[0] < S, t1 = kc0 <= tq0[1] + 15 && tq0[1] < S;
+        const bool t0 = kc0 <= tq0[0] + 15 && tq0[0] < S;
+        const bool t1 = NQT == 2 && kc0 <= tq0[NQT - 1] + 15 && tq0[NQT - 1] < S;
         if (t0 && t1)
-            compute(std::integral_constant<int, 3>{}, st, kc0);
+            compute(std::integral_constant<int, NQT == 2 ? 3 : 1>{}, st, kc0);
         else if (t1)
-            compute(std::integral_constant<int, 2>{}, st, kc0);
+            compute(std::integral_constant<int, NQT == 2 ? 2 : 1>{}, st, kc0);
         else if (t0)
             compute(std::integral_constant<int, 1>{}, st, kc0);
     };
@@ -622,7 +632,7 @@ __global__ __launch_bounds__(64 * kWaves2) __attribute__((amdgpu_waves_per_eu(2,
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no copy may land in LDS after the workgroup has gone
 
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
+    for (int qt = 0; qt < NQT; ++qt) {
         const float l = lacc[qt][0];   // every row of the tile holds the sum for query j
         const int qi = tq0[qt] + j;
         if (qi >= S)
@@ -646,16 +656,28 @@ int launch_dh128(const void *q, const void *kc, const void *vc, void *ctx, const
 {
     const float scale = (float)(_Float16)(1.0f / sqrtf(128.0f));
     dim3 grid(B * H, (S + kBQ2 - 1) / kBQ2);
-    if (alibi != nullptr)
-        hipLaunchKernelGGL((prefill_attention_dh128_kernel<true>), grid, dim3(64 * kWaves2), 0, st,
-                           static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(kc),
-                           static_cast<const _Float16 *>(vc), static_cast<_Float16 *>(ctx),
-                           static_cast<const _Float16 *>(alibi), pad, H, S, T_cap, scale);
-    else
-        hipLaunchKernelGGL((prefill_attention_dh128_kernel<false>), grid, dim3(64 * kWaves2), 0, st,
-                           static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(kc),
-                           static_cast<const _Float16 *>(vc), static_cast<_Float16 *>(ctx),
-                           static_cast<const _Float16 *>(alibi), pad, H, S, T_cap, scale);
+    // sixteen one-tile wavefronts for shorter prompts, eight two-tile wavefronts beyond (measured, B*H = 256: without
+    // a bias 3-8 % faster up to 4096 tokens and 1 % slower at 8192; with ALiBi equal up to 2048, 5-7 % slower
+    // beyond); a tuning override picks either
+    const int forced = eet::tuning().prefill_waves;
+    const bool wide = forced == 16 || (forced != 8 && S <= (alibi != nullptr ? 1024 : 4096));
+#define EET_PF_LAUNCH(A_, N_, W_)                                                                                  \
+    hipLaunchKernelGGL((prefill_attention_dh128_kernel<A_, N_, W_>), grid, dim3(64 * W_), 0, st,                    \
+                       static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(kc),                       \
+                       static_cast<const _Float16 *>(vc), static_cast<_Float16 *>(ctx),                           \
+                       static_cast<const _Float16 *>(alibi), pad, H, S, T_cap, scale)
+    if (alibi != nullptr) {
+        if (wide)
+            EET_PF_LAUNCH(true, 1, 16);
+        else
+            EET_PF_LAUNCH(true, 2, 8);
+    } else {
+        if (wide)
+            EET_PF_LAUNCH(false, 1, 16);
+        else
+            EET_PF_LAUNCH(false, 2, 8);
+    }
+#undef EET_PF_LAUNCH
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }

@@ -115,6 +115,16 @@ def test_prefill_attention_one_dominant_key(gpu, dh, dominant):
     assert_close(got, want, what=f"dominant key {dominant}")
 
 
+@pytest.mark.parametrize("waves", [8, 16])
+@pytest.mark.parametrize("S,use_pad,use_alibi", [(300, True, False), (1025, False, True), (64, False, False),
+                                                 (515, True, True)])
+def test_prefill_attention_wavefront_counts_dh128(gpu, tuning, waves, S, use_pad, use_alibi):
+    """Head size 128 runs with eight two-tile or sixteen one-tile wavefronts per workgroup depending on the prompt
+    length; both are forced here at lengths on either side of the switch and held to the same oracle."""
+    tuning("EET_PREFILL_WAVES", waves)
+    test_prefill_attention(gpu, 2, 2, S, 128, use_pad, use_alibi)
+
+
 @pytest.mark.parametrize("S,use_alibi", [(300, False), (130, True)])
 def test_prefill_attention_register_staged_kernel_dh128(gpu, tuning, S, use_alibi):
     """Head size 128 normally takes the DMA kernel; the register-staged one (the path of the other head

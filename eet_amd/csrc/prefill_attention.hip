@@ -345,7 +345,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 // ds_read_b64_tr_b16, which hands lane i column i of a 4 x 16 block of halves.
 // ---------------------------------------------------------------------------
 constexpr int kD = 128;
-constexpr int kBQ2 = 256, kStages = 4;
+
 constexpr int kStageVec = 2 * 1024 + 16;   // u32x4 per stage: K rows, V rows, bias row (+ padding)
 
 // Measured on MI355X with 8 wavefronts reading back to back: a 16-byte operand read (lane = row) runs at
@@ -357,19 +357,22 @@ __device__ __forceinline__ int row_swz(int r) { return ((r & 7) << 1) | ((r >> 3
 
 typedef short short4v __attribute__((ext_vector_type(4)));
 
-// NQT 16-query tiles per wavefront, WAVES wavefronts: 256 queries per workgroup either way.  <2, 8>: two wavefronts
-// per SIMD with 256 registers each, every K and V operand read feeds two tiles; <1, 16>: four wavefronts per SIMD,
-// twice the operand reads (the LDS has the room), faster on short prompts, where a workgroup sees few chunks and
-// its start-up and the diagonal chunks weigh more.
-template <bool ALIBI, int NQT, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4))) void prefill_attention_dh128_kernel(
+// NQT 16-query tiles per wavefront, WAVES wavefronts, STAGES chunk buffers: 16 NQT WAVES queries per workgroup.
+// <2, 8, 4>: two wavefronts per SIMD with 256 registers each, every K and V operand read feeds two tiles;
+// <1, 8, 2>: half the queries and half the ring, so that two workgroups fit a CU, four wavefronts per SIMD, twice
+// the operand reads per query (the LDS has the room).  launch_dh128 says which runs when.
+template <bool ALIBI, int NQT, int WAVES, int STAGES>
+__global__ __launch_bounds__(64 * WAVES)
+    __attribute__((amdgpu_waves_per_eu(STAGES == 2 ? 2 * WAVES / 4 : WAVES / 4, STAGES == 2 ? 2 * WAVES / 4 : WAVES / 4))) void prefill_attention_dh128_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_cache, const _Float16 *__restrict__ v_cache,
     _Float16 *__restrict__ ctx, const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, int H, int S,
     int T_cap, float scale)
 {
 #if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
     constexpr int DC = kD / 32, DT = kD / 16;
-    __shared__ u32x4 lds[kStages * kStageVec];
+    constexpr int kBQ2 = 16 * NQT * WAVES;   // queries per workgroup
+    constexpr int kGroup = STAGES / 2;       // chunks per barrier
+    __shared__ u32x4 lds[STAGES * kStageVec];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -393,7 +396,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVE
     const __amdgpu_buffer_rsrc_t ars = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<_Float16 *>(ALIBI ? alibi + (size_t)h * S : q), 0, ALIBI ? (unsigned)S * 2u : 0u, 0x00020000);
 
-    static_assert(NQT * WAVES == 16 && (NQT == 1 || NQT == 2), "256 queries per workgroup");
+    static_assert((NQT == 1 || NQT == 2) && 16 % WAVES == 0 && (STAGES == 2 || STAGES == 4), "launch shape");
     constexpr int KI = 16 / WAVES;   // DMA instructions per wavefront for the K rows of a chunk (and for the V rows)
     // the query tiles of this wavefront: one early, one late (the causal triangle is split evenly)
     int tq0[NQT];
@@ -605,7 +608,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVE
 
     auto chunk = [&](int c) {
         const int kc0 = k_begin + c * kBK;
-        const u32x4 *st = lds + (c % kStages) * kStageVec;
+        const u32x4 *st = lds + (c % STAGES) * kStageVec;
         const bool t0 = kc0 <= tq0[0] + 15 && tq0[0] < S;
         const bool t1 = NQT == 2 && kc0 <= tq0[NQT - 1] + 15 && tq0[NQT - 1] < S;
         if (t0 && t1)
@@ -615,19 +618,22 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVE
         else if (t0)
             compute(std::integral_constant<int, 1>{}, st, kc0);
     };
-    // Two chunks per barrier: while chunks 2i and 2i + 1 are multiplied, 2i + 2 and 2i + 3 are on their way
-    // into the other two stages.  (A chunk past the end reads rows >= S: zeros, no memory touched beyond
-    // the range; past k_end but below S it is a wasted copy.)
-    dma_chunk(0, k_begin);
-    dma_chunk(1, k_begin + kBK);
-    for (int i = 0; 2 * i < nchunks; ++i) {
-        // everything requested so far is this iteration's pair of chunks
+    // kGroup chunks per barrier (two with four stages, one with two): while one group is multiplied the next is on
+    // its way into the other half of the ring.  (A chunk past the end reads rows >= S: zeros, no memory touched
+    // beyond the range; past k_end but below S it is a wasted copy.)
+#pragma unroll
+    for (int gi = 0; gi < kGroup; ++gi)
+        dma_chunk(gi, k_begin + gi * kBK);
+    for (int c0 = 0; c0 < nchunks; c0 += kGroup) {
+        // everything requested so far is this iteration's group of chunks
         asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-        dma_chunk((2 * i + 2) % kStages, k_begin + (2 * i + 2) * kBK);   // these two stages were read in iteration i - 1
-        dma_chunk((2 * i + 3) % kStages, k_begin + (2 * i + 3) * kBK);
-        chunk(2 * i);
-        if (2 * i + 1 < nchunks)
-            chunk(2 * i + 1);
+#pragma unroll
+        for (int gi = 0; gi < kGroup; ++gi)   // these stages were read in the iteration before
+            dma_chunk((c0 + kGroup + gi) % STAGES, k_begin + (c0 + kGroup + gi) * kBK);
+#pragma unroll
+        for (int gi = 0; gi < kGroup; ++gi)
+            if (c0 + gi < nchunks)
+                chunk(c0 + gi);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no copy may land in LDS after the workgroup has gone
 
@@ -655,27 +661,32 @@ int launch_dh128(const void *q, const void *kc, const void *vc, void *ctx, const
                  int H, int S, int T_cap, hipStream_t st)
 {
     const float scale = (float)(_Float16)(1.0f / sqrtf(128.0f));
-    dim3 grid(B * H, (S + kBQ2 - 1) / kBQ2);
-    // sixteen one-tile wavefronts for shorter prompts, eight two-tile wavefronts beyond (measured, B*H = 256: without
-    // a bias 3-8 % faster up to 4096 tokens and 1 % slower at 8192; with ALiBi equal up to 2048, 5-7 % slower
-    // beyond); a tuning override picks either
-    const int forced = eet::tuning().prefill_waves;
-    const bool wide = forced == 16 || (forced != 8 && S <= (alibi != nullptr ? 1024 : 4096));
-#define EET_PF_LAUNCH(A_, N_, W_)                                                                                  \
-    hipLaunchKernelGGL((prefill_attention_dh128_kernel<A_, N_, W_>), grid, dim3(64 * W_), 0, st,                    \
+    // Launch shape by prompt length (measured at B*H = 256 .. 320):
+    //   1  128 queries per workgroup, eight one-tile wavefronts, two stages: two workgroups share a CU, so the
+    //      start-up, the diagonal chunks and the drain of one overlap the other's work -- up to 1536 tokens
+    //      (+13 % at 256, +20 % at 512, +6-9 % at 1024, +2-3 % at 1536; 3-6 % behind from 2048 on);
+    //   2  256 queries, eight two-tile wavefronts, four stages (every operand read feeds two tiles) -- beyond.
+    // (256 queries as sixteen one-tile wavefronts was within 2 % of shape 2 everywhere and is not kept.)
+    // A tuning override picks either.
+    int shape = eet::tuning().prefill_shape;
+    if (shape < 1 || shape > 2)
+        shape = S <= 1536 ? 1 : 2;
+#define EET_PF_LAUNCH(A_, N_, W_, S_)                                                                              \
+    hipLaunchKernelGGL((prefill_attention_dh128_kernel<A_, N_, W_, S_>),                                          \
+                       dim3(B * H, (S + 16 * N_ * W_ - 1) / (16 * N_ * W_)), dim3(64 * W_), 0, st,                \
                        static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(kc),                       \
                        static_cast<const _Float16 *>(vc), static_cast<_Float16 *>(ctx),                           \
                        static_cast<const _Float16 *>(alibi), pad, H, S, T_cap, scale)
     if (alibi != nullptr) {
-        if (wide)
-            EET_PF_LAUNCH(true, 1, 16);
+        if (shape == 1)
+            EET_PF_LAUNCH(true, 1, 8, 2);
         else
-            EET_PF_LAUNCH(true, 2, 8);
+            EET_PF_LAUNCH(true, 2, 8, 4);
     } else {
-        if (wide)
-            EET_PF_LAUNCH(false, 1, 16);
+        if (shape == 1)
+            EET_PF_LAUNCH(false, 1, 8, 2);
         else
-            EET_PF_LAUNCH(false, 2, 8);
+            EET_PF_LAUNCH(false, 2, 8, 4);
     }
 #undef EET_PF_LAUNCH
     EET_HIP_CHECK(hipGetLastError());

@@ -19,7 +19,7 @@ struct Tuning {
     int mmha_nsplit = 0, mmha_threads = 0, mmha_ring = 0;
     // EET_PREFILL_LEGACY = 1: head size 128 takes the register-staged prefill attention kernel
     int prefill_legacy = 0;
-    int prefill_waves = 0;   // 8 or 16: wavefronts per workgroup of the head-size-128 prefill attention kernel; 0 = by prompt length
+    int prefill_shape = 0;   // 1, 2: launch shape of the head-size-128 prefill attention kernel; 0 = by prompt length
 };
 
 const Tuning &tuning();

@@ -115,13 +115,14 @@ def test_prefill_attention_one_dominant_key(gpu, dh, dominant):
     assert_close(got, want, what=f"dominant key {dominant}")
 
 
-@pytest.mark.parametrize("waves", [8, 16])
+@pytest.mark.parametrize("shape", [1, 2])
 @pytest.mark.parametrize("S,use_pad,use_alibi", [(300, True, False), (1025, False, True), (64, False, False),
-                                                 (515, True, True)])
-def test_prefill_attention_wavefront_counts_dh128(gpu, tuning, waves, S, use_pad, use_alibi):
-    """Head size 128 runs with eight two-tile or sixteen one-tile wavefronts per workgroup depending on the prompt
-    length; both are forced here at lengths on either side of the switch and held to the same oracle."""
-    tuning("EET_PREFILL_WAVES", waves)
+                                                 (515, True, True), (1700, False, False)])
+def test_prefill_attention_launch_shapes_dh128(gpu, tuning, shape, S, use_pad, use_alibi):
+    """Head size 128 runs in one of two launch shapes (queries per workgroup, tiles per wavefront, ring depth)
+    depending on the prompt length; each is forced here at lengths on either side of the switch and held to
+    the same oracle."""
+    tuning("EET_PREFILL_SHAPE", shape)
     test_prefill_attention(gpu, 2, 2, S, 128, use_pad, use_alibi)
 
 

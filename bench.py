@@ -453,13 +453,15 @@ def prefill_gemm_bench(torch, eet, lib, dev, iters=10):
 
 
 def prefill_attention_bench(torch, lib, dev, iters=5):
-    """Causal prefill attention (flash-style MFMA kernel) at the prompt shapes of configurations 4 and 5:
-    TFLOP/s over the causal half of the work, 4 * B * H * (S^2 / 2) * dh."""
+    """Causal prefill attention (flash-style MFMA kernel) at the prompt shapes of configurations 4 and 5 (and one
+    long prompt): TFLOP/s over the causal half of the work, 4 * B * H * (S^2 / 2) * dh."""
     out = {}
     st = torch.cuda.current_stream()
     for name, B, H, S, alibi in (("llama7b B=8 H=32 S=1024", 8, 32, 1024, False),
                                  ("baichuan13b B=8 H=40 S=2048 alibi", 8, 40, 2048, True),
-                                 ("baichuan13b B=8 H=40 S=2048 no bias", 8, 40, 2048, False)):
+                                 ("baichuan13b B=8 H=40 S=2048 no bias", 8, 40, 2048, False),
+                                 # no configuration has a prompt this long: the kernel away from its diagonal chunks
+                                 ("long prompt B=1 H=32 S=8192 no bias", 1, 32, 8192, False)):
         dh = 128
         g = torch.Generator(device=dev).manual_seed(S)
         q, kc, vc = [torch.randn(B, H, S, dh, generator=g, device=dev).half() for _ in range(3)]

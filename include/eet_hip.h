@@ -51,6 +51,8 @@ int eet_packed_layout_version(void);
  * that run every kernel variant; value NULL or "" restores the table.  Keys:
  *   EET_GEMM_SMALL_M_CONFIG "nt,waves,u"       EET_GEMM_LARGE_M_TILE "tm,tn[,ksplit]"
  *   EET_MMHA_NSPLIT / EET_MMHA_THREADS / EET_MMHA_UNROLL "n"
+ *   EET_PREFILL_LEGACY "1" (register-staged prefill attention at head size 128)
+ *   EET_PREFILL_SHAPE "1" | "2" (launch shape of the head-size-128 prefill kernel)
  * An override naming a kernel variant that does not exist is ignored.  The same
  * keys are read from the environment once, at load, when EET_HIP_TUNING=1; no
  * launch reads the environment (the reference queries occupancy and runs its

@@ -134,9 +134,24 @@ def test_fused_argument_errors():
     from eet_amd._lib import lib
     buf = np.zeros(4096, np.uint8)
     p = buf.ctypes.data
-    L = lib()
+    L = _lib.lib()
     assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 7, None, None, 0.0, None, 0, None) == -1          # unknown epilogue
     assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 1, None, None, 0.0, None, 0, None) == -1          # residual missing
     assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 32, 64, 0, p, None, 0.0, None, 0, None) == -1             # residual without the epilogue
     assert L.eet_gemm_w8a16_fused(p, p, p, p, 1, 48, 64, 2, None, None, 0.0, None, 0, None) == -2          # odd tile count
     assert L.eet_gemm_w8a16_fused(p, p, p, p, 64, 32, 64, 0, None, p, 1e-6, None, 0, None) == -2       # RMSnorm prologue, M > 32
+
+
+def test_tuning_keys():
+    """Every documented tuning key is accepted and cleared (host state only, no GPU); malformed values and
+    unknown keys are refused with a message."""
+    L = _lib.lib()
+    for name, value in [("EET_GEMM_SMALL_M_CONFIG", "2,8,1"), ("EET_GEMM_LARGE_M_TILE", "4,4"),
+                        ("EET_GEMM_LARGE_M_TILE", "2,2,4"), ("EET_MMHA_NSPLIT", "2"), ("EET_MMHA_THREADS", "256"),
+                        ("EET_MMHA_UNROLL", "4"), ("EET_PREFILL_LEGACY", "1"), ("EET_PREFILL_SHAPE", "2")]:
+        assert L.eet_set_tuning(name.encode(), value.encode()) == 0, L.eet_last_error()
+        assert L.eet_set_tuning(name.encode(), None) == 0
+    assert L.eet_set_tuning(b"EET_GEMM_SMALL_M_CONFIG", b"2,8") != 0
+    assert b"nt,waves,u" in L.eet_last_error()
+    assert L.eet_set_tuning(b"EET_NO_SUCH_KEY", b"1") != 0
+    assert b"unknown key" in L.eet_last_error()

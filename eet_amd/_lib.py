@@ -83,7 +83,8 @@ def check(status, what=""):
         raise RuntimeError(f"[EET][ERROR] {what or 'libeet_hip'}: {msg} (status {status})")
     if DEBUG_SYNC:
         import torch
-        if not torch.cuda.is_available():
+        # no waiting while the stream records a HIP graph: a synchronisation there invalidates the capture
+        if not torch.cuda.is_available() or torch.cuda.is_current_stream_capturing():
             return
         try:
             torch.cuda.synchronize()

@@ -452,6 +452,7 @@ __global__ __launch_bounds__(64 * WAVES)
     };
 
     constexpr float kLog2e = 1.4426950408889634f;
+    constexpr float kLazy = 8.0f;   // in powers of two
     const float scale2 = scale * kLog2e;
     const int k_begin = (padb / kBK) * kBK;
     const int k_end = min(S, q0 + kBQ2);
@@ -535,9 +536,21 @@ __global__ __launch_bounds__(64 * WAVES)
             cmax = max_over_lane_groups(cmax);
             if (!ALIBI)
                 cmax *= scale2;
-            const float m_new = fmaxf(m_run[qt], cmax);
-            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-            const float corr = __builtin_amdgcn_exp2f(m_run[qt] - m_safe);  // 0 while nothing has been seen
+            // m_run is the reference exponent of the query: it follows the maximum lazily, only when a chunk's
+            // maximum passes it by more than kLazy (then the accumulators are rescaled; rare after a query's first
+            // chunk, where following every new maximum rescaled in most chunks of a short prompt).  Weights reach
+            // 2^kLazy at most, well inside fp16, and numerator and denominator share the reference.
+            const float m_ref = m_run[qt];
+            const bool raise = cmax > m_ref + kLazy;   // also the first keys of the query: m_ref is -inf
+            if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+                const float corr = raise ? __builtin_amdgcn_exp2f(m_ref - cmax) : 1.0f;   // 0 for the first keys
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    oacc[qt][dt] *= corr;
+                lacc[qt] *= corr;
+                m_run[qt] = raise ? cmax : m_ref;
+            }
+            const float m_safe = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];
             float p[4][4];
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
@@ -545,14 +558,6 @@ __global__ __launch_bounds__(64 * WAVES)
                 for (int r = 0; r < 4; ++r)
                     p[kt][r] = ALIBI ? __builtin_amdgcn_exp2f(sacc[qt][kt][r] - m_safe)
                                      : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qt][kt][r], scale2, -m_safe));
-            m_run[qt] = m_new;
-            // the accumulators are rescaled only when some query's maximum moved (rare after the first chunks)
-            if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-                    oacc[qt][dt] *= corr;
-                lacc[qt] *= corr;
-            }
 #pragma unroll
             for (int hf = 0; hf < 2; ++hf) {
                 half8 o;

@@ -115,6 +115,31 @@ def test_prefill_attention_one_dominant_key(gpu, dh, dominant):
     assert_close(got, want, what=f"dominant key {dominant}")
 
 
+@pytest.mark.parametrize("dh", [128, 64])
+@pytest.mark.parametrize("per_chunk", [0.5, 3.0, 7.0, 12.0])
+def test_prefill_attention_rising_scores(gpu, dh, per_chunk):
+    """Scores that rise along the keys by `per_chunk` powers of two per 64-key chunk: the running reference of the
+    softmax is passed by a little in every chunk (below and above the point where the kernel re-bases its
+    accumulators), by a lot in a few, and the weights of a row span the whole fp16 range.  Held to the oracle."""
+    B, H, S = 1, 2, 448
+    g = torch.Generator().manual_seed(int(per_chunk * 10) + dh)
+    unit = torch.ones(dh) / dh ** 0.5
+    q = (unit * 4.0 + torch.randn(B, H, S, dh, generator=g) * 0.05).half()
+    # q . k / sqrt(dh) = 4 a_t / sqrt(dh); in powers of two: times log2(e)
+    slope = per_chunk / 64.0 / 1.4427 * dh ** 0.5 / 4.0
+    a = torch.arange(S).float() * slope
+    k = (unit[None, None, None, :] * a[None, None, :, None] + torch.randn(B, H, S, dh, generator=g) * 0.05).half()
+    v = torch.randn(B, H, S, dh, generator=g).half()
+    want = O.prefill_attention(q.numpy(), k.numpy(), v.numpy(), None, None)
+    ctx = torch.empty(B, S, H * dh, dtype=torch.float16, device=gpu)
+    qd, kd, vd = q.to(gpu), k.to(gpu), v.to(gpu)
+    check(lib().eet_prefill_attention(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), ctx.data_ptr(), None, None,
+                                      B, H, S, dh, S, stream()))
+    got = ctx.cpu().numpy()
+    assert np.isfinite(got).all()
+    assert_close(got, want, what=f"rising scores {per_chunk}/chunk")
+
+
 @pytest.mark.parametrize("shape", [1, 2])
 @pytest.mark.parametrize("S,use_pad,use_alibi", [(300, True, False), (1025, False, True), (64, False, False),
                                                  (515, True, True), (1700, False, False)])

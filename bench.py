@@ -75,12 +75,28 @@ def fused_launch_weights(eet_ops, weights):
     return out
 
 
-def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup, probe=False, probe_grid_scale=1):
+def bench_lib():
+    """libeet_bench.so: the read-only streaming probe (measurement only, not part of the product ABI)."""
+    import ctypes
+    path = os.path.join(ROOT, "eet_amd", "libeet_bench.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with `python -m eet_amd.build`")
+    h = ctypes.CDLL(path)
+    vp, sz = ctypes.c_void_p, ctypes.c_size_t
+    h.eet_hbm_stream_probe.restype = ctypes.c_int
+    h.eet_hbm_stream_probe.argtypes = [vp, sz, ctypes.c_int, vp, sz, vp]
+    return h
+
+
+def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup, probe=False, probe_grid_scale=1, chained=False):
     """Returns seconds per step (one pass over all linears), measured with
     events on the stream the kernels are launched on.  Launches named in
     RMS_LAUNCHES carry the RMSnorm prologue, as in the decoder.  probe=True
     replaces every GEMM by the read-only streaming probe over the same weight
-    buffer with the same grid (the machine's ceiling for this launch chain)."""
+    buffer with the same grid (the machine's ceiling for this launch chain).
+    chained=True issues the pass as ONE chain (eet_gemm_w8a16_chained): every launch but the
+    first of a pass is enqueued without the queue barrier and waits in the kernel for its
+    predecessor's completion counter."""
     st = torch.cuda.current_stream()
     calls = []
     for layer in weights:
@@ -93,16 +109,26 @@ def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup, probe=Fals
     f = lib.eet_gemm_w8a16_fused
     sp = st.cuda_stream
 
-    if probe:
+    if chained:
+        fc = lib.eet_gemm_w8a16_chained
+
+        def one_pass():
+            mode = 1                       # EET_CHAIN_FIRST, then EET_CHAIN_NEXT
+            for (a, w, s, c, m, n, k, epi, res, gam) in calls:
+                rc = fc(a, w, s, c, m, n, k, epi, res, gam, 1e-6, mode, sp)
+                if rc:
+                    raise RuntimeError(lib.eet_last_error().decode())
+                mode = 2
+    elif probe:
         sink = outs["probe_sink"]
-        g = lib.eet_hbm_stream_probe
+        g = bench_lib().eet_hbm_stream_probe
 
         def one_pass():
             for (a, w, s, c, m, n, k, epi, res, gam) in calls:
                 # the grid the GEMM uses for this shape: 256 workgroups, 688 for the merged gate|up matrix
                 rc = g(w, k * n, (688 if epi == EPI_SWIGLU else 256) * probe_grid_scale, sink.data_ptr(), sink.numel(), sp)
                 if rc:
-                    raise RuntimeError(lib.eet_last_error().decode())
+                    raise RuntimeError("eet_hbm_stream_probe failed")
     else:
         def one_pass():
             for (a, w, s, c, m, n, k, epi, res, gam) in calls:
@@ -561,6 +587,7 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the M = 1..32 sweep")
+    ap.add_argument("--no-chain", action="store_true", help="skip the chained-launch form of the GEMM pass")
     ap.add_argument("--no-baichuan", action="store_true",
                     help="skip benchmark configuration 5: Baichuan-13B-shaped decoder (40 layers, ALiBi), batch 32, "
                          "prompt 2048, 256 greedy tokens (needs ~85 GB of HBM and about a minute)")
@@ -639,6 +666,25 @@ def main():
                      "frac_of_stream_ceiling": round(step_bytes / sec / (weight_bytes / probe_sec), 4)},
         "host_wall_ms_per_step": round(wall * 1e3, 4),
     }
+
+    # the same pass issued as one chain (eet_gemm_w8a16_chained): launches without the queue barrier that
+    # wait in the kernel for their producer.  `value` stays the ordinary launch path.
+    if not args.no_chain:
+        import ctypes
+        gave_up = ctypes.c_int(0)
+        chain = {}
+        for m in ((M,) if args.no_sweep else (1, 4, 8, 16, 32)):
+            s_c, _, _ = time_gemm_pass(torch, L, fused, acts, outs, m, max(3, args.steps // 2), 1, chained=True)
+            b = pass_bytes(fused, m)
+            chain[f"M={m}"] = {"GB/s": round(b / s_c / 1e9, 1), "pct_peak": round(100 * b / s_c / 1e9 / HBM_PEAK_GBS, 2),
+                               "avg_launch_us": round(s_c / launches * 1e6, 3)}
+        if L.eet_chain_status(ctypes.byref(gave_up), 1, torch.cuda.current_stream().cuda_stream):
+            raise RuntimeError(L.eet_last_error().decode())
+        chain["a_wait_gave_up"] = bool(gave_up.value)
+        chain["what"] = ("the same launches as one chain per pass: each launch after the first is enqueued without the "
+                         "queue barrier (hipExtAnyOrderLaunch), requests its first weight batches and then waits in the "
+                         "kernel (bounded) for the completion counter of the launch before it")
+        result["chained_pass"] = chain
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(3)

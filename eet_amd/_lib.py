@@ -27,6 +27,9 @@ SIGNATURES = {
     "eet_gemm_w8a16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _vp]),
     "eet_gemm_w8a16_workspace": (_sz, [_i, _i, _i, _i]),
     "eet_gemm_w8a16_fused": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _f, _vp, _sz, _vp]),
+    "eet_gemm_w8a16_small_m_shape": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "eet_gemm_w8a16_chained": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _f, _i, _vp]),
+    "eet_chain_status": (_i, [_vp, _i, _vp]),
     "eet_mmha_decode_workspace": (_sz, [_i, _i, _i, _i]),
     "eet_mmha_decode": (_i, [_vp, _vp, _vp, _l, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
     "eet_mmha_decode_static_capacity": (_sz, []),
@@ -46,7 +49,6 @@ SIGNATURES = {
     "eet_swiglu": (_i, [_vp, _vp, _i, _i, _vp]),
     "eet_residual_add": (_i, [_vp, _vp, _i, _i, _vp]),
     "eet_kv_cache_reorder": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "eet_hbm_stream_probe": (_i, [_vp, _sz, _i, _vp, _sz, _vp]),
     "eet_prefill_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
 }
 

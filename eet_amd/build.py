@@ -1,7 +1,9 @@
-"""Builds libeet_hip.so (HIP kernels + C ABI + host packer) for gfx950 with hipcc.
+"""Builds libeet_hip.so (HIP kernels + C ABI + host packer) and libeet_bench.so (the read-only
+streaming probe that bench.py times beside the GEMM pass; no part of the operator interface) for
+gfx950 with hipcc.
 
-Run as `python -m eet_amd.build`.  The library is built in-tree, next to this
-file, so that it travels with the source tree.
+Run as `python -m eet_amd.build`.  The libraries are built in-tree, next to this
+file, so that they travel with the source tree.
 """
 import os
 import subprocess
@@ -12,7 +14,11 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libeet_hip.so")
 
-SOURCES = ["packer.cc", "tuning.cc", "decode_ops.cc", "packer_device.hip", "gemm_w8a16.hip", "gemm_w8a16_large.hip", "mmha_decode.hip", "prefill_attention.hip", "glue.hip", "probe.hip"]
+BENCH_LIB = os.path.join(HERE, "libeet_bench.so")
+
+SOURCES = ["packer.cc", "tuning.cc", "decode_ops.cc", "chain.hip", "packer_device.hip", "gemm_w8a16.hip",
+           "gemm_w8a16_large.hip", "mmha_decode.hip", "prefill_attention.hip", "glue.hip"]
+BENCH_SOURCES = ["probe.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -27,7 +33,7 @@ def build(verbose=True):
     objs = []
     procs = []
     os.makedirs(os.path.join(HERE, "_obj"), exist_ok=True)
-    for src in SOURCES:
+    for src in SOURCES + BENCH_SOURCES:
         obj = os.path.join(HERE, "_obj", src + ".o")
         if src.endswith(".hip"):
             cmd = [HIPCC] + [f for f in FLAGS if f != "-shared"] + ["-x", "hip", "-c"]
@@ -49,10 +55,12 @@ def build(verbose=True):
             failed = True
     if failed:
         raise RuntimeError("hipcc failed")
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
+    for lib, srcs in ((LIB, SOURCES), (BENCH_LIB, BENCH_SOURCES)):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + \
+              [os.path.join(HERE, "_obj", src + ".o") for src in srcs]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
     return LIB
 
 

@@ -16,6 +16,7 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 // 4 biased bytes -> 4 fp16 values (q = u8 - 128), exact.
 __device__ __forceinline__ void widen4(uint32_t x, half2v &lo, half2v &hi)
@@ -53,6 +54,7 @@ struct GemmArgs {
     void *ws;  // optional fp32 workspace (split-k partial results)
     size_t ws_bytes;
     hipStream_t st;
+    int chain = 0;  // kChainOff / kChainFirst / kChainNext (chain.h; small-M kernel only)
 };
 
 // gemm_w8a16_large.hip: the MFMA-tile kernel for M > 32, and the workspace it can use.

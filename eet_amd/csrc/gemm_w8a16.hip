@@ -26,6 +26,9 @@
 // more accurate and inside the 1e-2 / 1e-3 tolerance against fp32).
 #include <hip/hip_runtime.h>
 
+#include <hip/hip_ext.h>
+
+#include "chain.h"
 #include "gemm_common.h"
 #include "tuning.h"
 
@@ -78,6 +81,49 @@ __device__ __forceinline__ void load_batch(Batch<NT, RG, U> &b, __amdgpu_buffer_
 #pragma unroll
         for (int r = 0; r < RG; ++r)
             b.a[u][r] = abase[r][valid ? (kt + u * WAVES) * 8 : 0];
+    if (RMS) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            b.gam[u] = gbase[valid ? (kt + u * WAVES) * 8 : 0];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+#endif
+
+// The two halves of load_batch on their own, for the chained kernel: its first weight
+// batches are requested before the wait for the producer, the activations after it.  The
+// activations go through a buffer resource with the sc1 bit (agent scope: served by the L2,
+// which the hardware keeps coherent across XCDs for such accesses, and never by a stale L1
+// line); a request that is not `valid` is moved out of range.
+#if defined(__HIP_DEVICE_COMPILE__)
+constexpr int kAgentScope = 16;   // aux bits of a buffer access: sc1
+template <int NT, int RG, int WAVES, int U>
+__device__ __forceinline__ void load_batch_w(Batch<NT, RG, U> &b, __amdgpu_buffer_rsrc_t wrsrc,
+                                             const unsigned (&wtile)[NT], int lane, int kt, bool valid)
+{
+    constexpr int kStream = 2;
+    const unsigned voff = valid ? (unsigned)lane * 16u : 0x80000000u;
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            b.w[u][t] = __builtin_bit_cast(
+                u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, voff, wtile[t] + (unsigned)(kt + u * WAVES) * 1024u,
+                                                             kStream));
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <int NT, int RG, int WAVES, int U, bool RMS>
+__device__ __forceinline__ void load_batch_a_chained(Batch<NT, RG, U> &b, __amdgpu_buffer_rsrc_t arsrc,
+                                                     const unsigned (&aoff)[RG], const u32x4 *gbase, int kt, bool valid)
+{
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int r = 0; r < RG; ++r)
+            b.a[u][r] = __builtin_bit_cast(
+                u32x4, __builtin_amdgcn_raw_buffer_load_b128(arsrc, valid ? aoff[r] : 0x80000000u,
+                                                             (unsigned)(kt + u * WAVES) * 128u, kAgentScope));
     if (RMS) {
 #pragma unroll
         for (int u = 0; u < U; ++u)
@@ -146,12 +192,15 @@ __device__ __forceinline__ void mma_batch(const Batch<NT, RG, U> &b, floatx4 (&a
 
 // NT: n-tiles per workgroup.  RG: groups of 8 activation rows (M <= 8 * RG).
 // RMS: RMSnorm prologue compiled in (it costs ~20-30 registers, so the plain
-// GEMM is a separate instantiation).
-template <int NT, int RG, int WAVES, int U, bool RMS>
+// GEMM is a separate instantiation).  CHAIN: the chained form (chain.h): the first two
+// weight batches are requested, then the workgroup waits for the producer of A and of the
+// residual rows, reads both with agent-scope loads, writes C with agent-scope stores and
+// signals its own completion; `link` is ignored otherwise.
+template <int NT, int RG, int WAVES, int U, bool RMS, bool CHAIN>
 __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
     _Float16 *__restrict__ C, int M, int N, int K, const _Float16 *__restrict__ residual, int epi,
-    const _Float16 *__restrict__ rms_gamma, float rms_eps)
+    const _Float16 *__restrict__ rms_gamma, float rms_eps, eet::ChainLink link)
 {
 #if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
     constexpr int MT = (RG + 1) / 2;
@@ -214,7 +263,7 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
             sc0[idx] = *reinterpret_cast<const half4 *>(scale + nt * 16 + 4 * g);
             if (epi == kEpiSwiglu)
                 sc1[idx] = *reinterpret_cast<const half4 *>(scale + min(nt + 1, ntiles - 1) * 16 + 4 * g);
-            if (epi == kEpiResidual) {
+            if (!CHAIN && epi == kEpiResidual) {
                 const int m = min(mt * 16 + j, M - 1);
                 res[idx] = *reinterpret_cast<const half4 *>(residual + (size_t)m * N + nt * 16 + 4 * g);
             }
@@ -240,26 +289,81 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     const int nbatch = mine / U;
     constexpr int STEP = U * WAVES;
     int kt = wave;
-    {
+    if constexpr (CHAIN) {
+        // Chained form.  The weights of the first two batches depend on nothing and are requested
+        // at once; then the wait for the producer; then the residual rows and the activations of
+        // those two batches.  From there on a batch is multiplied and its buffer refilled with the
+        // batch after next, so the wait before a multiply counts exactly the younger batch.
+        const unsigned a_bytes = (unsigned)M * (unsigned)K * 2u;
+        unsigned aoff[RG];
+#pragma unroll
+        for (int r = 0; r < RG; ++r)
+            aoff[r] = ((unsigned)min(8 * r + (lane >> 3), M - 1) * (unsigned)K + (unsigned)(lane & 7) * 8u) * 2u;
         Batch<NT, RG, U> b0, b1;
-        load_batch<NT, RG, WAVES, U, RMS>(b0, wrsrc, wtile, lane, abase, gbase, kt, nbatch > 0);
+        load_batch_w<NT, RG, WAVES, U>(b0, wrsrc, wtile, lane, kt, nbatch > 0);
+        load_batch_w<NT, RG, WAVES, U>(b1, wrsrc, wtile, lane, kt + STEP, nbatch > 1);
+        eet::chain_wait(link);
+        // the compiler must not know that these are the kernel's read-only arguments: what they
+        // point to has just been written by another kernel
+        const _Float16 *A_now = A, *res_now = residual;
+        asm volatile("" : "+s"(A_now), "+s"(res_now)::"memory");
+        const __amdgpu_buffer_rsrc_t arsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16 *>(A_now), 0, a_bytes, 0x00020000);
+        if (epi == kEpiResidual) {
+            const __amdgpu_buffer_rsrc_t rrsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<_Float16 *>(res_now), 0, (unsigned)M * (unsigned)N * 2u, 0x00020000);
+            int idx = 0;
+            for (int unit = wave; unit < units; unit += WAVES, ++idx) {
+                const int mt = unit % MT, t = unit / MT;
+                const int nt = min(nt0 + t, ntiles - 1), m = min(mt * 16 + j, M - 1);
+                const unsigned off = ((unsigned)m * (unsigned)N + (unsigned)(nt * 16 + 4 * g)) * 2u;
+                res[idx] = __builtin_bit_cast(half4, __builtin_amdgcn_raw_buffer_load_b64(rrsrc, off, 0, kAgentScope));
+            }
+        }
+        load_batch_a_chained<NT, RG, WAVES, U, RMS>(b0, arsrc, aoff, gbase, kt, nbatch > 0);
+        load_batch_a_chained<NT, RG, WAVES, U, RMS>(b1, arsrc, aoff, gbase, kt + STEP, nbatch > 1);
         int i = 0;
         for (; i + 2 <= nbatch; i += 2) {
-            load_batch<NT, RG, WAVES, U, RMS>(b1, wrsrc, wtile, lane, abase, gbase, kt + STEP, true);
             mma_batch<NT, RG, U, RMS>(b0, acc, slab, lane, ss);
-            load_batch<NT, RG, WAVES, U, RMS>(b0, wrsrc, wtile, lane, abase, gbase, kt + 2 * STEP, i + 2 < nbatch);
+            load_batch_w<NT, RG, WAVES, U>(b0, wrsrc, wtile, lane, kt + 2 * STEP, i + 2 < nbatch);
+            load_batch_a_chained<NT, RG, WAVES, U, RMS>(b0, arsrc, aoff, gbase, kt + 2 * STEP, i + 2 < nbatch);
             mma_batch<NT, RG, U, RMS>(b1, acc, slab, lane, ss);
+            load_batch_w<NT, RG, WAVES, U>(b1, wrsrc, wtile, lane, kt + 3 * STEP, i + 3 < nbatch);
+            load_batch_a_chained<NT, RG, WAVES, U, RMS>(b1, arsrc, aoff, gbase, kt + 3 * STEP, i + 3 < nbatch);
             kt += 2 * STEP;
         }
         if (i < nbatch) {
             mma_batch<NT, RG, U, RMS>(b0, acc, slab, lane, ss);
             kt += STEP;
         }
-    }
-    for (; kt < ktiles; kt += WAVES) {
-        Batch<NT, RG, 1> b;
-        load_batch<NT, RG, WAVES, 1, RMS>(b, wrsrc, wtile, lane, abase, gbase, kt, true);
-        mma_batch<NT, RG, 1, RMS>(b, acc, slab, lane, ss);
+        for (; kt < ktiles; kt += WAVES) {
+            Batch<NT, RG, 1> b;
+            load_batch_w<NT, RG, WAVES, 1>(b, wrsrc, wtile, lane, kt, true);
+            load_batch_a_chained<NT, RG, WAVES, 1, RMS>(b, arsrc, aoff, gbase, kt, true);
+            mma_batch<NT, RG, 1, RMS>(b, acc, slab, lane, ss);
+        }
+    } else {
+        {
+            Batch<NT, RG, U> b0, b1;
+            load_batch<NT, RG, WAVES, U, RMS>(b0, wrsrc, wtile, lane, abase, gbase, kt, nbatch > 0);
+            int i = 0;
+            for (; i + 2 <= nbatch; i += 2) {
+                load_batch<NT, RG, WAVES, U, RMS>(b1, wrsrc, wtile, lane, abase, gbase, kt + STEP, true);
+                mma_batch<NT, RG, U, RMS>(b0, acc, slab, lane, ss);
+                load_batch<NT, RG, WAVES, U, RMS>(b0, wrsrc, wtile, lane, abase, gbase, kt + 2 * STEP, i + 2 < nbatch);
+                mma_batch<NT, RG, U, RMS>(b1, acc, slab, lane, ss);
+                kt += 2 * STEP;
+            }
+            if (i < nbatch) {
+                mma_batch<NT, RG, U, RMS>(b0, acc, slab, lane, ss);
+                kt += STEP;
+            }
+        }
+        for (; kt < ktiles; kt += WAVES) {
+            Batch<NT, RG, 1> b;
+            load_batch<NT, RG, WAVES, 1, RMS>(b, wrsrc, wtile, lane, abase, gbase, kt, true);
+            mma_batch<NT, RG, 1, RMS>(b, acc, slab, lane, ss);
+        }
     }
 
     // RMSnorm prologue: each wavefront's share of sum(x^2) per row.  Lanes
@@ -295,6 +399,15 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
             s += red[(w * NT * MT + tile) * 64 + lane];
         return s;
     };
+    // four output halves of one lane; the chained form stores them write-through (agent scope)
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc(
+        C, 0, (unsigned)M * (unsigned)(epi == kEpiSwiglu ? N / 2 : N) * 2u, 0x00020000);
+    auto store_out = [&](half4 o, size_t elem) {
+        if constexpr (CHAIN)
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, o), crsrc, (unsigned)elem * 2u, 0, kAgentScope);
+        else
+            *reinterpret_cast<half4 *>(C + elem) = o;
+    };
     int idx = 0;
     for (int unit = wave; unit < units; unit += WAVES, ++idx) {
         const int mt = unit % MT;
@@ -321,7 +434,7 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
                     o[r] = (_Float16)(up * gate / (1.0f + __expf(-gate)));
                 }
                 const int n = ((nt0 + t) / 2) * 16 + 4 * g;
-                *reinterpret_cast<half4 *>(C + (size_t)m * (N / 2) + n) = o;
+                store_out(o, (size_t)m * (N / 2) + n);
             }
         } else {
             const int t = unit / MT;
@@ -334,10 +447,12 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
                     o[r] = (_Float16)(s[r] * (float)sc0[idx][r] * inv);
                 if (epi == kEpiResidual)
                     o = o + res[idx];  // fp16 add of the rounded product, like the separate kernel
-                *reinterpret_cast<half4 *>(C + (size_t)m * N + n) = o;
+                store_out(o, (size_t)m * N + n);
             }
         }
     }
+    if constexpr (CHAIN)
+        eet::chain_signal(link);
 #endif
 }
 
@@ -350,8 +465,30 @@ int launch_small_m(const GemmArgs &a)
 {
     const int ntiles = a.N / 16;
     dim3 grid((ntiles + NT - 1) / NT), block(WAVES * 64);
-    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U, RMS>), grid, block, 0, a.st, a.A, a.Wp, a.scale, a.C, a.M,
-                       a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps);
+    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U, RMS, false>), grid, block, 0, a.st, a.A, a.Wp, a.scale,
+                       a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, eet::ChainLink{});
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
+// The chained form: the first launch of a chain is an ordinary launch that signals; a later
+// one is issued without the queue barrier and waits in the kernel for its predecessor.
+template <int NT, int RG, int WAVES, int U, bool RMS>
+int launch_small_m_chained(const GemmArgs &a)
+{
+    const int ntiles = a.N / 16;
+    dim3 grid((ntiles + NT - 1) / NT), block(WAVES * 64);
+    eet::ChainLink link;
+    bool any_order = false;
+    if (int rc = eet::chain_link("eet_gemm_w8a16_chained", a.chain, grid.x, a.st, &link, &any_order))
+        return rc;
+    auto kern = w8a16_small_m_kernel<NT, RG, WAVES, U, RMS, true>;
+    if (any_order)
+        hipExtLaunchKernelGGL(kern, grid, block, 0, a.st, nullptr, nullptr, hipExtAnyOrderLaunch, a.A, a.Wp, a.scale,
+                              a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, link);
+    else
+        hipLaunchKernelGGL(kern, grid, block, 0, a.st, a.A, a.Wp, a.scale, a.C, a.M, a.N, a.K, a.residual, a.epi,
+                           a.rms_gamma, a.rms_eps, link);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
@@ -368,27 +505,46 @@ constexpr bool small_m_fits(int nt, int rg, int waves, int u)
     return stage <= 65536 && red <= 147456 && batch_vgprs <= (waves == 16 ? 96 : 200);
 }
 
+// Internal status of dispatch_small_m: no instantiation for this (nt, waves, u) at this row
+// count / prologue.  Never crosses the C ABI.
+constexpr int kNoVariant = 1;
+
+// Runs the instantiation named by cfg, or with dry = true only tells whether it exists
+// (EET_OK / kNoVariant) without launching anything.
 template <int RG>
-int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a)
+int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a, bool dry)
 {
-#define EET_CASE(NT_, W_, U_)                                      \
-    if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_) {         \
-        if constexpr (small_m_fits(NT_, RG, W_, U_))               \
-            return launch_small_m<NT_, RG, W_, U_, false>(a);      \
+#define EET_CASE(NT_, W_, U_)                                                         \
+    if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_) {                            \
+        if constexpr (small_m_fits(NT_, RG, W_, U_))                                  \
+            return dry ? EET_OK : launch_small_m<NT_, RG, W_, U_, false>(a);          \
     }
-#define EET_CASE_RMS(NT_, W_, U_)                                  \
-    if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_) {         \
-        if constexpr (small_m_fits(NT_, RG, W_, U_))               \
-            return launch_small_m<NT_, RG, W_, U_, true>(a);       \
+#define EET_CASE_RMS(NT_, W_, U_)                                                     \
+    if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_) {                            \
+        if constexpr (small_m_fits(NT_, RG, W_, U_))                                  \
+            return dry ? EET_OK : launch_small_m<NT_, RG, W_, U_, true>(a);           \
+    }
+    if (a.chain != eet::kChainOff) {
+        // chained kernels exist for the launch shapes pick_small_m can return
+#define EET_CASE_CHAIN(NT_, W_, U_)                                                              \
+    if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_) {                                        \
+        if constexpr (small_m_fits(NT_, RG, W_, U_))                                              \
+            return dry ? EET_OK                                                                   \
+                       : (a.rms_gamma ? launch_small_m_chained<NT_, RG, W_, U_, true>(a)          \
+                                      : launch_small_m_chained<NT_, RG, W_, U_, false>(a));       \
+    }
+        EET_CASE_CHAIN(1, 8, 2) EET_CASE_CHAIN(1, 16, 2) EET_CASE_CHAIN(1, 16, 1)
+        EET_CASE_CHAIN(2, 8, 2) EET_CASE_CHAIN(2, 8, 1) EET_CASE_CHAIN(3, 8, 1)
+        EET_CASE_CHAIN(4, 8, 1) EET_CASE_CHAIN(6, 8, 1) EET_CASE_CHAIN(8, 8, 1)
+#undef EET_CASE_CHAIN
+        return kNoVariant;
     }
     if (a.rms_gamma != nullptr) {
         // the launch shapes pick_small_m can return
         EET_CASE_RMS(1, 8, 2) EET_CASE_RMS(1, 16, 2) EET_CASE_RMS(1, 16, 1)
         EET_CASE_RMS(2, 8, 2) EET_CASE_RMS(2, 8, 1) EET_CASE_RMS(3, 8, 1)
         EET_CASE_RMS(4, 8, 1) EET_CASE_RMS(6, 8, 1) EET_CASE_RMS(8, 8, 1)
-        return eet::fail(EET_ERR_INVALID_ARGUMENT,
-                         "eet_gemm_w8a16_fused: no RMSnorm-prologue kernel for nt=%d waves=%d u=%d", cfg.nt,
-                         cfg.waves, cfg.u);
+        return kNoVariant;
     }
     EET_CASE(1, 4, 4) EET_CASE(1, 8, 4) EET_CASE(1, 16, 4) EET_CASE(1, 8, 2) EET_CASE(1, 16, 2) EET_CASE(1, 16, 1)
     EET_CASE(2, 4, 2) EET_CASE(2, 8, 2) EET_CASE(2, 16, 2) EET_CASE(2, 8, 4) EET_CASE(2, 16, 1) EET_CASE(2, 8, 1)
@@ -397,8 +553,7 @@ int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a)
     EET_CASE(6, 8, 1) EET_CASE(8, 8, 1)
 #undef EET_CASE_RMS
 #undef EET_CASE
-    return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no small-M kernel for nt=%d waves=%d u=%d (M=%d)",
-                     cfg.nt, cfg.waves, cfg.u, a.M);
+    return kNoVariant;
 }
 
 // Shape -> launch shape: the number of n-tiles per workgroup (NT) that minimises
@@ -447,25 +602,40 @@ SmallMConfig pick_small_m(int M, int N, int K, int epi, bool rms)
     return SmallMConfig{best_nt, 8, 1};
 }
 
+int dispatch_by_rows(SmallMConfig cfg, const GemmArgs &a, bool dry)
+{
+    if (a.M <= 8)
+        return dispatch_small_m<1>(cfg, a, dry);
+    if (a.M <= 16)
+        return dispatch_small_m<2>(cfg, a, dry);
+    return dispatch_small_m<4>(cfg, a, dry);
+}
+
+// The launch shape a call runs with: the tuning override when an instantiation of that shape
+// exists for this call (decided without launching), otherwise the table's choice.
+SmallMConfig resolve_small_m(const GemmArgs &a)
+{
+    const eet::Tuning &tune = eet::tuning();
+    if (tune.has_small_m && (a.epi != kEpiSwiglu || tune.small_m_nt % 2 == 0)) {
+        const SmallMConfig forced{tune.small_m_nt, tune.small_m_waves, tune.small_m_u};
+        if (dispatch_by_rows(forced, a, true) == EET_OK)
+            return forced;
+    }
+    return pick_small_m(a.M, a.N, a.K, a.epi, a.rms_gamma != nullptr);
+}
+
 int run_small_m(const GemmArgs &a)
 {
     // the kernel addresses the packed weights through one buffer resource with 32-bit offsets
     if ((size_t)a.K * a.N >= (1ull << 31))
         return eet::fail(EET_ERR_UNSUPPORTED_SHAPE, "eet_gemm_w8a16: K x N = %d x %d exceeds the 2 GiB weight limit",
                          a.K, a.N);
-    auto dispatch = [&](SmallMConfig cfg) {
-        if (a.M <= 8)
-            return dispatch_small_m<1>(cfg, a);
-        if (a.M <= 16)
-            return dispatch_small_m<2>(cfg, a);
-        return dispatch_small_m<4>(cfg, a);
-    };
-    // a tuning override runs when such a kernel exists for this call; otherwise the table decides
-    const eet::Tuning &tune = eet::tuning();
-    if (tune.has_small_m && (a.epi != kEpiSwiglu || tune.small_m_nt % 2 == 0) &&
-        dispatch(SmallMConfig{tune.small_m_nt, tune.small_m_waves, tune.small_m_u}) == EET_OK)
-        return EET_OK;
-    return dispatch(pick_small_m(a.M, a.N, a.K, a.epi, a.rms_gamma != nullptr));
+    const SmallMConfig cfg = resolve_small_m(a);
+    const int rc = dispatch_by_rows(cfg, a, false);   // a launch failure is returned as it is
+    if (rc == kNoVariant)
+        return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no small-M kernel for nt=%d waves=%d u=%d (M=%d%s)",
+                         cfg.nt, cfg.waves, cfg.u, a.M, a.rms_gamma ? ", RMSnorm prologue" : "");
+    return rc;
 }
 
 }  // namespace
@@ -531,6 +701,21 @@ extern "C" int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *sc
                              kEpiNone, nullptr, 0.f, workspace, workspace_bytes, static_cast<hipStream_t>(stream)});
 }
 
+extern "C" int eet_gemm_w8a16_small_m_shape(int M, int N, int K, int epilogue, int rms_prologue, int *nt, int *waves,
+                                            int *k_tiles_per_batch)
+{
+    EET_REQUIRE(nt && waves && k_tiles_per_batch, EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16_small_m_shape: null pointer");
+    EET_REQUIRE(M >= 1 && M <= 32 && N > 0 && K > 0 && K % 64 == 0 && N % 16 == 0, EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_gemm_w8a16_small_m_shape: not a shape the small-M kernel takes (M=%d N=%d K=%d)", M, N, K);
+    GemmArgs a{};
+    a.M = M, a.N = N, a.K = K, a.epi = epilogue;
+    static const _Float16 kSomeGamma = 0;
+    a.rms_gamma = rms_prologue ? &kSomeGamma : nullptr;   // only tested against null
+    const SmallMConfig cfg = resolve_small_m(a);
+    *nt = cfg.nt, *waves = cfg.waves, *k_tiles_per_batch = cfg.u;
+    return EET_OK;
+}
+
 extern "C" size_t eet_gemm_w8a16_workspace(int M, int N, int K, int epilogue)
 {
     if (M <= 32 || N <= 0 || K <= 0 || K % 64 != 0 || N % 16 != 0)
@@ -538,29 +723,50 @@ extern "C" size_t eet_gemm_w8a16_workspace(int M, int N, int K, int epilogue)
     return eet::large_m_workspace(M, N, K, epilogue);
 }
 
+static int gemm_fused(const char *fn, const void *A, const void *Wpacked, const void *scale, void *C, int M, int N,
+                      int K, int epilogue, const void *residual, const void *rms_gamma, float rms_eps,
+                      void *workspace, size_t workspace_bytes, int chain, void *stream)
+{
+    if (int rc = check_gemm_args(fn, A, Wpacked, scale, C, M, N, K))
+        return rc;
+    EET_REQUIRE(epilogue == EET_EPILOGUE_NONE || epilogue == EET_EPILOGUE_RESIDUAL || epilogue == EET_EPILOGUE_SWIGLU,
+                EET_ERR_INVALID_ARGUMENT, "%s: unknown epilogue %d", fn, epilogue);
+    EET_REQUIRE((epilogue == EET_EPILOGUE_RESIDUAL) == (residual != nullptr), EET_ERR_INVALID_ARGUMENT,
+                "%s: residual must be given exactly for EET_EPILOGUE_RESIDUAL", fn);
+    EET_REQUIRE(residual == nullptr || reinterpret_cast<uintptr_t>(residual) % 8 == 0, EET_ERR_INVALID_ARGUMENT,
+                "%s: residual must be 8-byte aligned", fn);
+    EET_REQUIRE(epilogue != EET_EPILOGUE_SWIGLU || N % 32 == 0, EET_ERR_UNSUPPORTED_SHAPE,
+                "%s: the SwiGLU epilogue needs N %% 32 == 0 (gate/up tile pairs), got N=%d", fn, N);
+    EET_REQUIRE(rms_gamma == nullptr || (M <= 32 && reinterpret_cast<uintptr_t>(rms_gamma) % 16 == 0),
+                EET_ERR_UNSUPPORTED_SHAPE,
+                "%s: the RMSnorm prologue is available for M <= 32 only (M=%d) and needs a 16-byte aligned gamma", fn,
+                M);
+    EET_REQUIRE(chain == eet::kChainOff || chain == eet::kChainFirst || chain == eet::kChainNext,
+                EET_ERR_INVALID_ARGUMENT, "%s: unknown chain mode %d", fn, chain);
+    EET_REQUIRE(chain == eet::kChainOff || (M >= 1 && M <= 32), EET_ERR_UNSUPPORTED_SHAPE,
+                "%s: chained launches exist for 1 <= M <= 32 only (M=%d)", fn, M);
+    if (M == 0)
+        return EET_OK;
+    GemmArgs args{static_cast<const _Float16 *>(A), static_cast<const u32x4 *>(Wpacked),
+                  static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(C), M, N, K,
+                  static_cast<const _Float16 *>(residual), epilogue, static_cast<const _Float16 *>(rms_gamma), rms_eps,
+                  workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+    args.chain = chain;
+    return run_gemm(args);
+}
+
 extern "C" int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, void *C, int M, int N,
                                     int K, int epilogue, const void *residual, const void *rms_gamma, float rms_eps,
                                     void *workspace, size_t workspace_bytes, void *stream)
 {
-    if (int rc = check_gemm_args("eet_gemm_w8a16_fused", A, Wpacked, scale, C, M, N, K))
-        return rc;
-    EET_REQUIRE(epilogue == EET_EPILOGUE_NONE || epilogue == EET_EPILOGUE_RESIDUAL || epilogue == EET_EPILOGUE_SWIGLU,
-                EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16_fused: unknown epilogue %d", epilogue);
-    EET_REQUIRE((epilogue == EET_EPILOGUE_RESIDUAL) == (residual != nullptr), EET_ERR_INVALID_ARGUMENT,
-                "eet_gemm_w8a16_fused: residual must be given exactly for EET_EPILOGUE_RESIDUAL");
-    EET_REQUIRE(residual == nullptr || reinterpret_cast<uintptr_t>(residual) % 8 == 0, EET_ERR_INVALID_ARGUMENT,
-                "eet_gemm_w8a16_fused: residual must be 8-byte aligned");
-    EET_REQUIRE(epilogue != EET_EPILOGUE_SWIGLU || N % 32 == 0, EET_ERR_UNSUPPORTED_SHAPE,
-                "eet_gemm_w8a16_fused: the SwiGLU epilogue needs N %% 32 == 0 (gate/up tile pairs), got N=%d", N);
-    EET_REQUIRE(rms_gamma == nullptr || (M <= 32 && reinterpret_cast<uintptr_t>(rms_gamma) % 16 == 0),
-                EET_ERR_UNSUPPORTED_SHAPE,
-                "eet_gemm_w8a16_fused: the RMSnorm prologue is available for M <= 32 only (M=%d) and needs a "
-                "16-byte aligned gamma", M);
-    if (M == 0)
-        return EET_OK;
-    return run_gemm(GemmArgs{static_cast<const _Float16 *>(A), static_cast<const u32x4 *>(Wpacked),
-                             static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(C), M, N, K,
-                             static_cast<const _Float16 *>(residual), epilogue,
-                             static_cast<const _Float16 *>(rms_gamma), rms_eps, workspace, workspace_bytes,
-                             static_cast<hipStream_t>(stream)});
+    return gemm_fused("eet_gemm_w8a16_fused", A, Wpacked, scale, C, M, N, K, epilogue, residual, rms_gamma, rms_eps,
+                      workspace, workspace_bytes, eet::kChainOff, stream);
+}
+
+extern "C" int eet_gemm_w8a16_chained(const void *A, const void *Wpacked, const void *scale, void *C, int M, int N,
+                                      int K, int epilogue, const void *residual, const void *rms_gamma, float rms_eps,
+                                      int chain, void *stream)
+{
+    return gemm_fused("eet_gemm_w8a16_chained", A, Wpacked, scale, C, M, N, K, epilogue, residual, rms_gamma, rms_eps,
+                      nullptr, 0, chain, stream);
 }

@@ -90,8 +90,11 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
     // Replayable form (a launch recorded into a HIP graph): the step lives in device
     // memory, rope_row is the base of the whole rotary table and the bias rows have a
     // fixed leading dimension, so that the same recorded arguments serve every step.
+    // `step` arrives as step_max, the largest step the recording was sized for (launch
+    // shape, rotary table rows, bias leading dimension): a step outside [1, step_max]
+    // is clamped into it, so that no replay reads past those.
     if (step_dev != nullptr) {
-        step = min(max(*step_dev, 1), T_cap);
+        step = min(max(*step_dev, 1), min(step, T_cap));
         if (rope_row != nullptr)
             rope_row += (size_t)(step - 1) * DH;
     }

@@ -5,9 +5,11 @@
 // the same grids as the GEMM pass: what it reaches is what this machine allows a
 // chain of dependent launches of those sizes, i.e. the practical ceiling the
 // GEMM's HBM rate is to be read against (next to the published 8 TB/s).
+// No counterpart in the reference and no part of the operator interface.
 #include <hip/hip_runtime.h>
 
-#include "common.h"
+#include <cstddef>
+#include <cstdint>
 
 namespace {
 
@@ -60,18 +62,15 @@ __global__ __launch_bounds__(kThreads) void hbm_stream_probe_kernel(const u32x4 
 
 }  // namespace
 
+// Built into libeet_bench.so, not into the product library: bench.py binds it directly.
+// Returns 0, or -1 for bad arguments, -3 for a failed launch.
 extern "C" int eet_hbm_stream_probe(const void *src, size_t bytes, int workgroups, void *sink, size_t sink_bytes,
                                     void *stream)
 {
-    EET_REQUIRE(src && sink, EET_ERR_INVALID_ARGUMENT, "eet_hbm_stream_probe: null pointer");
-    EET_REQUIRE(workgroups > 0 && workgroups <= 65536 && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
-                    reinterpret_cast<uintptr_t>(sink) % 16 == 0,
-                EET_ERR_INVALID_ARGUMENT, "eet_hbm_stream_probe: bad grid or alignment");
-    EET_REQUIRE(sink_bytes >= (size_t)workgroups * 1024, EET_ERR_WORKSPACE,
-                "eet_hbm_stream_probe: sink needs 1 KiB per workgroup (%zu bytes), %zu given", (size_t)workgroups * 1024,
-                sink_bytes);
+    if (!src || !sink || workgroups <= 0 || workgroups > 65536 || reinterpret_cast<uintptr_t>(src) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(sink) % 16 != 0 || sink_bytes < (size_t)workgroups * 1024)
+        return -1;   // sink: 1 KiB of device memory per workgroup
     hipLaunchKernelGGL(hbm_stream_probe_kernel, dim3(workgroups), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
                        static_cast<const u32x4 *>(src), bytes / 16, static_cast<u32x4 *>(sink));
-    EET_HIP_CHECK(hipGetLastError());
-    return EET_OK;
+    return hipGetLastError() == hipSuccess ? 0 : -3;
 }

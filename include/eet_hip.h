@@ -53,6 +53,8 @@ int eet_packed_layout_version(void);
  *   EET_MMHA_NSPLIT / EET_MMHA_THREADS / EET_MMHA_UNROLL "n"
  *   EET_PREFILL_LEGACY "1" (register-staged prefill attention at head size 128)
  *   EET_PREFILL_SHAPE "1" | "2" (launch shape of the head-size-128 prefill kernel)
+ *   EET_DECODE_CHAIN "1" (eet_mmha_int8_decode / eet_gated_ffn_int8_decode chain their launches)
+ *   EET_CHAIN_SPIN_LIMIT "n" / EET_CHAIN_SLEEP "n" (bounded wait of a chained launch)
  * An override naming a kernel variant that does not exist is ignored.  The same
  * keys are read from the environment once, at load, when EET_HIP_TUNING=1; no
  * launch reads the environment (the reference queries occupancy and runs its
@@ -151,6 +153,48 @@ int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, 
                          const void *rms_gamma, float rms_eps, void *workspace,
                          size_t workspace_bytes, void *stream);
 
+/* The launch shape the small-M kernel (1 <= M <= 32) runs a call with: n-tiles per
+ * workgroup, wavefronts per workgroup, k-tiles per register batch -- the tuning
+ * override EET_GEMM_SMALL_M_CONFIG when a kernel of that shape exists for the
+ * call, otherwise the table's choice.  For sweeps and for tests that must know
+ * which variant ran.  The reference's counterpart is the CutlassGemmConfig its
+ * heuristic returns (cutlass_heuristic.cc:106-207). */
+int eet_gemm_w8a16_small_m_shape(int M, int N, int K, int epilogue, int rms_prologue, int *nt,
+                                 int *waves, int *k_tiles_per_batch);
+
+/* Chained launches (1 <= M <= 32): eet_gemm_w8a16_fused for a sequence of launches
+ * in which each reads what the previous one wrote -- the decode step of
+ * csrc/op/llama_mmha.cpp:202-266 and csrc/op/gated_ffn_int8.cpp:98-132, which the
+ * reference issues as serial launches on one stream.
+ *   EET_CHAIN_FIRST  an ordinary launch (ordered behind all earlier work of the
+ *                    stream) that also publishes a completion counter.
+ *   EET_CHAIN_NEXT   enqueued without the queue's barrier: the kernel may start
+ *                    while earlier launches of the stream still run, requests its
+ *                    first weight batches, and then waits IN THE KERNEL for the
+ *                    completion counter of the previous chained launch (which must
+ *                    have been made on the same stream of the same device) before it
+ *                    reads A or the residual rows.
+ * Contract of a NEXT launch: everything it reads was written by the previous
+ * chained launch or earlier, and no other work that it depends on, or that
+ * depends on it, is enqueued on the stream between the two.  Ordinary launches
+ * that follow a chain are ordered behind all of it as usual.  Outputs are written
+ * with agent-scope stores and inputs read with agent-scope loads (coherent across
+ * the XCDs' L2 caches); results are bit-identical to eet_gemm_w8a16_fused.
+ * The wait is bounded: after EET_CHAIN_SPIN_LIMIT polls (eet_set_tuning; default
+ * 65536, about 20 ms) a workgroup gives up, sets a device error word and goes on,
+ * so that every kernel exits; the results of the chain are then undefined and
+ * eet_chain_status reports it.  Not for streams that are being captured into a
+ * HIP graph (refused).  A GPU that other processes or streams keep busy can delay
+ * a producer for longer than the bound: chain only on a GPU the caller owns. */
+enum { EET_CHAIN_OFF = 0, EET_CHAIN_FIRST = 1, EET_CHAIN_NEXT = 2 };
+int eet_gemm_w8a16_chained(const void *A, const void *Wpacked, const void *scale, void *C,
+                           int M, int N, int K, int epilogue, const void *residual,
+                           const void *rms_gamma, float rms_eps, int chain, void *stream);
+
+/* Waits for `stream`, then *gave_up = 1 if any chained wait on the current device
+ * has given up since the word was last cleared (0 otherwise); clear != 0 resets it. */
+int eet_chain_status(int *gave_up, int clear, void *stream);
+
 /* Masked multi-head decode attention for one new token per sequence.
  *   dh        32, 64, 96 or 128, the head sizes the reference instantiates
  *   q, k, v   [B][H][dh] half; with qkv_stride != 0 they are rows of a fused
@@ -186,7 +230,11 @@ int eet_mmha_decode(const void *q, const void *k, const void *v, long qkv_stride
  * whose B*H*nsplit*(dh+2)*4 bytes exceed the capacity (only reachable through a
  * tuning override) fails with EET_ERR_WORKSPACE.  All calls on one GPU share the
  * array: calls that overlap in time on different streams of one GPU race;
- * nothing needs clearing between calls. */
+ * nothing needs clearing between calls.  The first call on each GPU looks the
+ * array's device address up (hipGetSymbolAddress, a runtime query that may load
+ * the code object): make that first call OUTSIDE a stream capture (one warm call
+ * per device; eet_mmha_decode_static_capacity() does not count, it touches no
+ * device).  `stream` must belong to the device that is current at the call. */
 size_t eet_mmha_decode_static_capacity(void);
 int eet_mmha_decode_static(const void *q, const void *k, const void *v, long qkv_stride,
                            void *k_cache, void *v_cache, void *ctx, const void *alibi,
@@ -277,7 +325,9 @@ int eet_prefill_attention(const void *q, const void *k_cache, const void *v_cach
  * for every token).  What changes from step to step lives in device memory:
  *   step_dev    int32 in device memory: the step of this call (rows attended,
  *               the new token included); eet_step_advance(step_dev, 1, stream)
- *               recorded ahead of the layers moves it on at each replay
+ *               recorded ahead of the layers moves it on at each replay.  The
+ *               kernel clamps the value it reads into [1, step_max]: a replay past
+ *               step_max repeats step_max instead of reading past the tables
  *   step_max    the largest step the recording will be replayed at (<= T_cap):
  *               launch shape and workspace are chosen for it
  *   rope_table  NULL or the BASE of the eet_rope_table table (>= step_max rows):
@@ -301,16 +351,6 @@ int eet_mmha_int8_decode_replayable(const void *x, const void *rms_gamma, float 
                                     int B, int H, int dh, int hidden, const int *step_dev,
                                     int step_max, int T_cap, void *workspace, size_t workspace_bytes,
                                     void *stream);
-
-/* Measurement utility (no counterpart in the reference): reads `bytes` of device
- * memory once with the access pattern and launch structure of the small-M GEMM
- * (contiguous range per workgroup, 128-bit non-temporal loads, one reduction and
- * one small store per workgroup) and nothing else.  Launched over the same
- * buffers, in the same order and with the same grids as a GEMM pass, it measures
- * the HBM rate this machine allows such a chain of dependent launches.  sink: 1 KiB
- * of device memory per workgroup. */
-int eet_hbm_stream_probe(const void *src, size_t bytes, int workgroups, void *sink,
-                         size_t sink_bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -571,8 +571,8 @@ def recorded_traffic(M, layers):
             continue
         m = re.search(rf"traffic_bytes_per_launch M={M} layers={layers}: (\d+)", text)
         if m:
-            return int(m.group(1))
-    return None
+            return int(m.group(1)), os.path.relpath(path, ROOT)
+    return None, None
 
 
 def main():
@@ -638,6 +638,9 @@ def main():
                                    probe_grid_scale=sc)[0] for sc in (1, 2, 4))
     weight_bytes = sum(w.numel() for layer in fused for (w, _, _) in layer.values())
     ceiling_gbs = weight_bytes / probe_sec / 1e9
+    traffic, traffic_file = recorded_traffic(M, args.layers)
+    traffic_source = (f"{traffic_file}: FETCH_SIZE + WRITE_SIZE of this command under rocprofv3 --pmc, recorded when that "
+                      "file was committed; NOT measured in this run (counters need the profiler)") if traffic_file else None
     result = {
         "metric": "int8 W-only GEMM HBM GB/s (% peak) at M=1..16; LLaMA-7B int8 decode tokens/s, 1 GPU",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -656,7 +659,7 @@ def main():
                      "algorithmic_bytes_per_launch": round(step_bytes / launches),
                      # HBM-side bytes per launch, from the committed rocprofv3 --pmc summary of this workload
                      # (FETCH_SIZE and WRITE_SIZE scaled by a copy kernel of known size); null if none matches
-                     "traffic": recorded_traffic(M, args.layers),
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "stream_ceiling": {"GB/s": round(ceiling_gbs, 1), "frac_of_peak": round(ceiling_gbs / HBM_PEAK_GBS, 4),
                                         "ms_per_step": round(probe_sec * 1e3, 4),
                                         "what": "the same 128 launches per step as read-only streams of the same weight "

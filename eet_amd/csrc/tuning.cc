@@ -46,8 +46,6 @@ int apply(const char *name, const char *value)
         slot = &t.prefill_legacy;
     else if (std::strcmp(name, "EET_PREFILL_SHAPE") == 0)
         slot = &t.prefill_shape;
-    else if (std::strcmp(name, "EET_DECODE_CHAIN") == 0)
-        slot = &t.decode_chain;
     else if (std::strcmp(name, "EET_CHAIN_SLEEP") == 0)
         slot = &t.chain_sleep;
     else if (std::strcmp(name, "EET_CHAIN_SPIN_LIMIT") == 0) {
@@ -69,7 +67,7 @@ struct EnvInit {
             return;
         for (const char *name : {"EET_GEMM_SMALL_M_CONFIG", "EET_GEMM_LARGE_M_TILE", "EET_MMHA_NSPLIT",
                                  "EET_MMHA_THREADS", "EET_MMHA_UNROLL", "EET_PREFILL_LEGACY", "EET_PREFILL_SHAPE",
-                                 "EET_DECODE_CHAIN", "EET_CHAIN_SLEEP", "EET_CHAIN_SPIN_LIMIT"})
+                                 "EET_CHAIN_SLEEP", "EET_CHAIN_SPIN_LIMIT"})
             if (const char *v = std::getenv(name))
                 if (apply(name, v) != EET_OK)
                     std::fprintf(stderr, "[EET][WARN] %s\n", eet::last_error_slot().c_str());

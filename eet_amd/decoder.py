@@ -200,8 +200,17 @@ class Int8Decoder:
         """Records one incremental step (step counter advance, embedding, all layers, final norm,
         lm_head, argmax, feeding the token back) into a HIP graph, after a prompt has been
         processed eagerly.  next_ids [B] are the tokens the first replay consumes.  Returns a
-        function that replays the step and returns the new tokens [B] (a static buffer)."""
+        function that replays the step and returns the new tokens [B] (a static buffer).
+
+        The graph holds raw device pointers.  Everything they point to is kept alive with the
+        graph (the named workspaces handed out while recording, the KV caches, the static
+        input / output buffers); a replay refuses to run when a layer's cache tensors are no
+        longer the recorded ones (a beam reorder swaps them), and brings the device-side step
+        back in line when eager calls or a new prompt moved the host-side step in between."""
         cfg, dev = self.cfg, self.embed.device
+        if self.reorder_state is not None and self.reorder_state.numel() != 0:
+            raise RuntimeError("[EET][ERROR] capture_decode_step: a decoder that reorders its KV cache (beam search) "
+                               "cannot replay a recorded step: the reorder swaps the cache buffers the graph points to")
         B = next_ids.shape[0]
         lib = ops.lib()
         step_dev = torch.tensor([self.layers[0][0].step], dtype=torch.int32, device=dev)
@@ -215,32 +224,53 @@ class Int8Decoder:
             out_tok.copy_(torch.argmax(logits[:, -1, :], dim=-1))
             ids.copy_(out_tok[:, None])
         try:
-            # eager warm-up on a side stream (allocates every workspace), then undone: the cache row it
-            # wrote is written again by the first replay
-            keep = ids.clone()
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side), torch.no_grad():
-                one_step()
-                ops.check(lib.eet_step_advance(step_dev.data_ptr(), -1, ops._stream()), "eet_step_advance")
-                ids.copy_(keep)
-            torch.cuda.current_stream().wait_stream(side)
-            self._shift_host_steps(-1)
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph), torch.no_grad():
-                one_step()
-            self._shift_host_steps(-1)      # recording ran the host code once; no kernel has run
+            with ops.workspaces.recording() as handed:
+                # eager warm-up on a side stream (allocates every workspace), then undone: the cache row it
+                # wrote is written again by the first replay
+                keep = ids.clone()
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side), torch.no_grad():
+                    one_step()
+                    ops.check(lib.eet_step_advance(step_dev.data_ptr(), -1, ops._stream()), "eet_step_advance")
+                    ids.copy_(keep)
+                torch.cuda.current_stream().wait_stream(side)
+                self._shift_host_steps(-1)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph), torch.no_grad():
+                    one_step()
+                self._shift_host_steps(-1)      # recording ran the host code once; no kernel has run
         finally:
             ops.replay_state = None
+        caches = [(attn.k_cache, attn.v_cache) for attn, _ in self.layers]
+        state = {"step": self.layers[0][0].step}     # what step_dev holds
 
-        def replay():
-            if self.layers[0][0].step + 1 > cfg.max_full_seq:
-                raise RuntimeError(f"[EET][ERROR] decode step {self.layers[0][0].step + 1} exceeds max_full_seq "
+        def replay(next_ids=None):
+            """One recorded step.  next_ids [B]: the tokens to consume instead of the previous replay's output
+            (needed after eager calls or a new prompt on this decoder)."""
+            host_step = self.layers[0][0].step
+            if host_step + 1 > cfg.max_full_seq:
+                raise RuntimeError(f"[EET][ERROR] decode step {host_step + 1} exceeds max_full_seq "
                                    f"{cfg.max_full_seq}")
+            if self.reorder_state is not None and self.reorder_state.numel() != 0:
+                raise RuntimeError("[EET][ERROR] replay: reorder_state is set; a recorded step cannot reorder the cache")
+            for (attn, _), (k, v) in zip(self.layers, caches):
+                if attn.k_cache is not k or attn.v_cache is not v:
+                    raise RuntimeError("[EET][ERROR] replay: a layer's KV cache is no longer the buffer this step was "
+                                       "recorded with (beam reorder?): record the step again")
+            if any(attn.step != host_step for attn, _ in self.layers):
+                raise RuntimeError("[EET][ERROR] replay: the layers disagree about the current step")
+            if host_step != state["step"]:
+                # eager calls or a new prompt moved the host-side step since the last replay
+                step_dev.fill_(host_step)
+            if next_ids is not None:
+                ids.copy_(next_ids.reshape(B, 1))
             graph.replay()
             self._shift_host_steps(1)
+            state["step"] = host_step + 1
             return out_tok
-        self._graph_keep = (graph, step_dev, ids, out_tok)
+        self._graph_keep = (graph, step_dev, ids, out_tok, handed, caches)
+        replay.keep = self._graph_keep      # the closure owns what the graph points to
         return replay
 
     @torch.no_grad()

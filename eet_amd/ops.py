@@ -58,6 +58,7 @@ class _StreamScope:
 class _Workspaces:
     def __init__(self):
         self._bufs = {}
+        self._recorders = []
 
     def get(self, name, numel, dtype, device):
         key = (name, str(device), dtype)
@@ -65,10 +66,29 @@ class _Workspaces:
         if buf is None or buf.numel() < numel:
             buf = torch.empty(max(int(numel), 1), dtype=dtype, device=device)
             self._bufs[key] = buf
+        for handed in self._recorders:
+            handed.append(buf)
         return buf
 
     def clear(self):
         self._bufs.clear()
+
+    def recording(self):
+        """Context manager that collects every buffer handed out inside it.  A HIP graph records raw
+        device pointers: whoever records one keeps the collected tensors alive for as long as the
+        graph lives, so that a later, larger request under the same name (which replaces the named
+        buffer) or clear() cannot hand the recorded memory back to the allocator."""
+        ws = self
+
+        class _Rec:
+            def __enter__(self):
+                self.handed = []
+                ws._recorders.append(self.handed)
+                return self.handed
+
+            def __exit__(self, *a):
+                ws._recorders.remove(self.handed)
+        return _Rec()
 
 
 workspaces = _Workspaces()

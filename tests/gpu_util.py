@@ -22,6 +22,23 @@ def assert_close(got, want, rtol=RTOL, atol=ATOL, what=""):
     assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.size} outside tolerance, max err {err.max():.5f}"
 
 
+def measured(got, want, what, bound=None, rtol=RTOL):
+    """Error of one fused launch, printed and -- with `bound` -- asserted: `excess` is the largest
+    err - rtol * |want| over the elements, i.e. the absolute tolerance the launch needs at the
+    north-star's relative tolerance.  `bound` is 1.5 x the excess observed on an MI355X (at least the
+    north-star's 1e-3 is always allowed); returns (max_abs_err, excess)."""
+    got = np.asarray(got, dtype=np.float32)
+    want = np.asarray(want, dtype=np.float32)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    err = np.abs(got - want)
+    excess = float((err - rtol * np.abs(want)).max())
+    print(f"ERR {what}: max_abs_err {err.max():.3e} needs atol {max(excess, 0.0):.3e} at rtol {rtol:g}"
+          + (f" (bound {bound:.1e})" if bound is not None else ""), flush=True)
+    if bound is not None:
+        assert excess <= bound, f"{what}: needs atol {excess:.3e} at rtol {rtol:g}, bound {bound:.1e}"
+    return float(err.max()), excess
+
+
 def gemm_workspace(M, N, K, epi, device, min_bytes=0):
     """(pointer, bytes) of the optional split-k workspace the library asks for
     (None, 0 when it asks for none); min_bytes forces a larger one for tests

@@ -15,7 +15,7 @@ import torch
 import eet_amd
 from oracle import ops as O
 
-from gpu_util import assert_close, gemm, gemm_fused
+from gpu_util import assert_close, gemm, gemm_fused, measured
 
 pytestmark = pytest.mark.gpu
 
@@ -56,6 +56,10 @@ def test_config3_gate_up_swiglu(gpu):
     assert_close(got, want, rtol=1e-2, atol=1e-3, what="config 3 gate|up")
 
 
+# absolute tolerance each fused launch may need at 1e-2 relative: 1.5 x what an MI355X run showed
+BOUNDS = {}
+
+
 def _rms_f32(x, gamma, eps):
     x32 = x.numpy().astype(np.float32)
     return x32 / np.sqrt((x32 * x32).mean(-1, keepdims=True) + np.float32(eps)) * gamma.numpy().astype(np.float32)
@@ -79,6 +83,7 @@ def test_config5_decode_linears(gpu, M):
     print(f"config 5 qkv+rmsnorm M={M}", flush=True)
     got = gemm_fused(xd, p.to(gpu), s.to(gpu), M, 3 * HIDDEN, HIDDEN, 0, None, gd, eps).cpu().numpy()
     want = xn @ (u.numpy().astype(np.float32) * s.numpy().astype(np.float32)[None, :])
+    measured(got, want, f"config5 rmsnorm+qkv M={M}", BOUNDS.get(("qkv", M)))
     assert_close(got, want, rtol=1e-2, atol=2e-3, what="qkv")
 
     # O + residual: 5120 -> 5120
@@ -87,6 +92,7 @@ def test_config5_decode_linears(gpu, M):
     print(f"config 5 o+residual M={M}", flush=True)
     got = gemm_fused(ctx.to(gpu), p.to(gpu), s.to(gpu), M, HIDDEN, HIDDEN, 1, xd).cpu().numpy()
     want = O.residual_add(O.dequant_matmul(ctx.numpy(), u.numpy(), s.numpy()), x.numpy())
+    measured(got, want, f"config5 o+residual M={M}", BOUNDS.get(("o", M)))
     assert_close(got, want, rtol=1e-2, atol=2e-3, what="o")
 
     # gate|up with the RMSnorm prologue and the SwiGLU epilogue: 5120 -> 27392
@@ -97,6 +103,7 @@ def test_config5_decode_linears(gpu, M):
     got = gemm_fused(xd, w01.to(gpu), s01.to(gpu), M, 2 * DFF, HIDDEN, 2, None, gd, eps).cpu().numpy()
     gate = xn @ (ug.numpy().astype(np.float32) * sg.numpy().astype(np.float32)[None, :])
     up = xn @ (uu.numpy().astype(np.float32) * su.numpy().astype(np.float32)[None, :])
+    measured(got, up * gate / (1 + np.exp(-gate)), f"config5 rmsnorm+gate|up+swiglu M={M}", BOUNDS.get(("gate|up", M)))
     assert_close(got, up * gate / (1 + np.exp(-gate)), rtol=1e-2, atol=3e-3, what="gate|up")
 
     # down + residual: 13696 -> 5120
@@ -105,4 +112,5 @@ def test_config5_decode_linears(gpu, M):
     print(f"config 5 down+residual M={M}", flush=True)
     got = gemm_fused(act.to(gpu), p.to(gpu), s.to(gpu), M, HIDDEN, DFF, 1, xd).cpu().numpy()
     want = O.residual_add(O.dequant_matmul(act.numpy(), u.numpy(), s.numpy()), x.numpy())
+    measured(got, want, f"config5 down+residual M={M}", BOUNDS.get(("down", M)))
     assert_close(got, want, rtol=1e-2, atol=2e-3, what="down")

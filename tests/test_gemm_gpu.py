@@ -134,6 +134,9 @@ def test_small_m_launch_shapes(gpu, tuning, cfg):
         assert_close(got, up * gate / (1 + np.exp(-gate)), rtol=1e-2, atol=3e-3, what=f"{cfg} rms+swiglu M={M}")
 
 
+# absolute tolerance the RMSnorm-prologue launches may need at 1e-2 relative: 1.5 x what an MI355X run showed
+PROLOGUE_BOUNDS = {}
+
 LARGE_M_TILES = ["8,4", "4,5", "4,4", "4,2", "2,2"]   # m-tiles, n-tiles per wavefront
 
 
@@ -330,6 +333,8 @@ def test_rmsnorm_prologue(gpu, M, K, N, epi):
     got = fused(x.to(gpu), p.to(gpu), s.to(gpu), M, N, K, epi, rd, gamma.to(gpu), eps).cpu().numpy()
     # the SwiGLU epilogue adds the fp16 roundings of gate and up (as the separate kernels have them)
     atol = 3e-3 if epi == 2 else 2e-3
+    from gpu_util import measured
+    measured(got, want, f"rmsnorm prologue M={M} K={K} N={N} epi={epi}", PROLOGUE_BOUNDS.get((M, K, N, epi)))
     assert_close(got, want, rtol=1e-2, atol=atol)
     # and the unfused path (eet_rmsnorm then the GEMM) agrees with the same reference
     from eet_amd._lib import check, lib

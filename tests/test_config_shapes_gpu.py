@@ -6,8 +6,8 @@ Configuration 3: the prefill GEMMs at M = 2048 (QKV 5120 -> 15360, O 5120 -> 512
 picks there, every output element compared.
 Configuration 5: the decode linears at M = 32 as the decoder ops launch them (RMSnorm prologue on
 QKV and gate|up, SwiGLU epilogue, residual epilogue on O and down).
-Tolerance: 1e-2 relative / 1e-3 absolute against dequantise-then-matmul in fp32 (absolute 2e-3 /
-3e-3 where a fused prologue / epilogue moves an fp16 rounding, as stated at each check)."""
+Tolerance: 1e-2 relative / 1e-3 absolute against dequantise-then-matmul in fp32; the fused decode
+launches are held to per-launch absolute bounds of 1.5 x their measured need (BOUNDS below)."""
 import numpy as np
 import pytest
 import torch
@@ -56,8 +56,19 @@ def test_config3_gate_up_swiglu(gpu):
     assert_close(got, want, rtol=1e-2, atol=1e-3, what="config 3 gate|up")
 
 
-# absolute tolerance each fused launch may need at 1e-2 relative: 1.5 x what an MI355X run showed
-BOUNDS = {}
+# Absolute tolerance each fused launch may need at 1e-2 relative: 1.5 x the need observed on an MI355X
+# (in brackets), and the north-star's 1e-3 wherever the observed need is below it.  Only the launches
+# that compare against a composition with NO intermediate fp16 rounding need more: the RMSnorm prologue
+# rounds x * gamma where the unfused path rounds x * gamma / rms, and the SwiGLU epilogue rounds gate and
+# up to fp16 (as the separate GEMMs would) before multiplying them.
+BOUNDS = {("qkv", 32): 1.6e-3,      # [1.06e-3]
+          ("qkv", 8): 1e-3,         # [9.7e-4]
+          ("o", 32): 1e-3,          # [5.9e-4]
+          ("o", 8): 1e-3,           # [2.8e-5]
+          ("gate|up", 32): 4.4e-3,  # [2.93e-3]
+          ("gate|up", 8): 3.2e-3,   # [2.11e-3]
+          ("down", 32): 1e-3,       # [9.8e-5]
+          ("down", 8): 1e-3}        # [6.5e-4]
 
 
 def _rms_f32(x, gamma, eps):
@@ -68,8 +79,8 @@ def _rms_f32(x, gamma, eps):
 @pytest.mark.parametrize("M", [32, 8])
 def test_config5_decode_linears(gpu, M):
     """The four launches of a Baichuan-13B decoder layer at batch 32 (and 8), with their fused parts.
-    The RMSnorm prologue is compared with the composition without an intermediate rounding (absolute
-    tolerance 2e-3; 3e-3 with SwiGLU on top, whose gate and up are rounded to fp16 first)."""
+    The RMSnorm prologue is compared with the composition without an intermediate rounding; the error of
+    every launch is printed and held to the per-launch bound of BOUNDS at 1e-2 relative."""
     from eet_amd.ops import interleave_gate_up
     g = torch.Generator().manual_seed(50 + M)
     eps = 1e-6
@@ -84,7 +95,6 @@ def test_config5_decode_linears(gpu, M):
     got = gemm_fused(xd, p.to(gpu), s.to(gpu), M, 3 * HIDDEN, HIDDEN, 0, None, gd, eps).cpu().numpy()
     want = xn @ (u.numpy().astype(np.float32) * s.numpy().astype(np.float32)[None, :])
     measured(got, want, f"config5 rmsnorm+qkv M={M}", BOUNDS.get(("qkv", M)))
-    assert_close(got, want, rtol=1e-2, atol=2e-3, what="qkv")
 
     # O + residual: 5120 -> 5120
     u, p, s = weights(HIDDEN, HIDDEN, 6)
@@ -93,7 +103,6 @@ def test_config5_decode_linears(gpu, M):
     got = gemm_fused(ctx.to(gpu), p.to(gpu), s.to(gpu), M, HIDDEN, HIDDEN, 1, xd).cpu().numpy()
     want = O.residual_add(O.dequant_matmul(ctx.numpy(), u.numpy(), s.numpy()), x.numpy())
     measured(got, want, f"config5 o+residual M={M}", BOUNDS.get(("o", M)))
-    assert_close(got, want, rtol=1e-2, atol=2e-3, what="o")
 
     # gate|up with the RMSnorm prologue and the SwiGLU epilogue: 5120 -> 27392
     ug, pg, sg = weights(HIDDEN, DFF, 7)
@@ -104,7 +113,6 @@ def test_config5_decode_linears(gpu, M):
     gate = xn @ (ug.numpy().astype(np.float32) * sg.numpy().astype(np.float32)[None, :])
     up = xn @ (uu.numpy().astype(np.float32) * su.numpy().astype(np.float32)[None, :])
     measured(got, up * gate / (1 + np.exp(-gate)), f"config5 rmsnorm+gate|up+swiglu M={M}", BOUNDS.get(("gate|up", M)))
-    assert_close(got, up * gate / (1 + np.exp(-gate)), rtol=1e-2, atol=3e-3, what="gate|up")
 
     # down + residual: 13696 -> 5120
     u, p, s = weights(DFF, HIDDEN, 9)
@@ -113,4 +121,3 @@ def test_config5_decode_linears(gpu, M):
     got = gemm_fused(act.to(gpu), p.to(gpu), s.to(gpu), M, HIDDEN, DFF, 1, xd).cpu().numpy()
     want = O.residual_add(O.dequant_matmul(act.numpy(), u.numpy(), s.numpy()), x.numpy())
     measured(got, want, f"config5 down+residual M={M}", BOUNDS.get(("down", M)))
-    assert_close(got, want, rtol=1e-2, atol=2e-3, what="down")

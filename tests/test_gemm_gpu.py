@@ -135,7 +135,13 @@ def test_small_m_launch_shapes(gpu, tuning, cfg):
 
 
 # absolute tolerance the RMSnorm-prologue launches may need at 1e-2 relative: 1.5 x what an MI355X run showed
-PROLOGUE_BOUNDS = {}
+# (in brackets); 1e-3, the north-star's, wherever the observed need is below it
+PROLOGUE_BOUNDS = {(1, 256, 64, 0): 1e-3,          # [3.5e-6]
+                   (8, 4096, 12288, 0): 1e-3,      # [8.0e-4]
+                   (8, 4096, 22016, 2): 3.3e-3,    # [2.16e-3]  SwiGLU: gate and up are rounded to fp16 first
+                   (16, 1024, 176, 0): 1e-3,       # [3.0e-4]
+                   (32, 512, 96, 2): 1e-3,         # [6.4e-5]
+                   (5, 11008, 4096, 1): 2.0e-3}    # [1.30e-3]  K = 11008 behind one moved rounding
 
 LARGE_M_TILES = ["8,4", "4,5", "4,4", "4,2", "2,2"]   # m-tiles, n-tiles per wavefront
 
@@ -303,8 +309,8 @@ def test_rmsnorm_prologue(gpu, M, K, N, epi):
 
     The fused kernel rounds x * gamma to fp16 and applies 1/rms to the fp32 sum; the unfused path
     rounds x * gamma / rms to fp16.  Both carry one fp16 rounding per activation, at different
-    places, so the comparison is against the composition with NO intermediate rounding, with the
-    absolute tolerance doubled to 2e-3 for that one rounding (relative stays 1e-2)."""
+    places, so the comparison is against the composition with NO intermediate rounding; the error is
+    printed and held to 1.5 x the need measured on an MI355X (PROLOGUE_BOUNDS; relative stays 1e-2)."""
     from eet_amd.ops import interleave_gate_up
     g = torch.Generator().manual_seed(M + K + N)
     x = (torch.randn(M, K, generator=g) * 1.7).half()
@@ -332,10 +338,9 @@ def test_rmsnorm_prologue(gpu, M, K, N, epi):
     rd = res.to(gpu) if res is not None else None
     got = fused(x.to(gpu), p.to(gpu), s.to(gpu), M, N, K, epi, rd, gamma.to(gpu), eps).cpu().numpy()
     # the SwiGLU epilogue adds the fp16 roundings of gate and up (as the separate kernels have them)
-    atol = 3e-3 if epi == 2 else 2e-3
     from gpu_util import measured
-    measured(got, want, f"rmsnorm prologue M={M} K={K} N={N} epi={epi}", PROLOGUE_BOUNDS.get((M, K, N, epi)))
-    assert_close(got, want, rtol=1e-2, atol=atol)
+    atol = PROLOGUE_BOUNDS[(M, K, N, epi)]
+    measured(got, want, f"rmsnorm prologue M={M} K={K} N={N} epi={epi}", atol)
     # and the unfused path (eet_rmsnorm then the GEMM) agrees with the same reference
     from eet_amd._lib import check, lib
     from gpu_util import stream
@@ -343,4 +348,5 @@ def test_rmsnorm_prologue(gpu, M, K, N, epi):
     xnd = torch.empty_like(xd)
     check(lib().eet_rmsnorm(xd.data_ptr(), gd.data_ptr(), xnd.data_ptr(), M, K, eps, stream()))
     got2 = fused(xnd, p.to(gpu), s.to(gpu), M, N, K, epi, rd).cpu().numpy()
-    assert_close(got2, want, rtol=1e-2, atol=atol)
+    # (this path rounds x * gamma / rms to fp16 before the GEMM: one rounding more than the reference form)
+    assert_close(got2, want, rtol=1e-2, atol=3e-3 if epi == 2 else 2e-3)

@@ -45,6 +45,9 @@ SIGNATURES = {
     "eet_gated_ffn_int8_decode": (_i, [_vp, _vp, _f] + [_vp] * 6 + [_i] * 4 + [_vp]),
     "eet_rope_table": (_i, [_vp, _i, _i, _vp]),
     "eet_rmsnorm": (_i, [_vp, _vp, _vp, _i, _i, _f, _vp]),
+    "eet_layernorm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
+    "eet_add_bias_residual_norm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
+    "eet_add_bias": (_i, [_vp, _vp, _i, _i, _vp]),
     "eet_qkv_split": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "eet_swiglu": (_i, [_vp, _vp, _i, _i, _vp]),
     "eet_residual_add": (_i, [_vp, _vp, _i, _i, _vp]),

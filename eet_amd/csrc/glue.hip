@@ -70,6 +70,112 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(const _Float16 *_
 }
 
 // ---------------------------------------------------------------------------
+// The bias / LayerNorm branch of the ops.  One kernel: y = x [+ residual] [+ bias] with the
+// reference's fp16 adds, then LayerNorm (gamma, beta: fp32 mean, then fp32 variance of the
+// centred values, (y - mean) * rsqrt(var + eps) * gamma + beta, one rounding) or, with beta
+// == nullptr, RMSnorm.  Covers decoder_norm1_kernel_opt<half> (csrc/core/layer_norm.cu:
+// 384-446), add_bias_input_layernorm<half> (:39-80) and add_input_RMSnorm<half> (:103-131).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kNormThreads) void add_norm_kernel(const _Float16 *x,   // may be `out` (in place)
+                                                                const _Float16 *__restrict__ residual,
+                                                                const _Float16 *__restrict__ bias,
+                                                                const _Float16 *__restrict__ gamma,
+                                                                const _Float16 *__restrict__ beta,
+                                                                _Float16 *out, int N, float eps)
+{
+    __shared__ float red[2][kNormThreads / 64];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const int nvec = N / 8;
+    const uint4 *xr = reinterpret_cast<const uint4 *>(x + (size_t)row * N);
+    const uint4 *rr = residual ? reinterpret_cast<const uint4 *>(residual + (size_t)row * N) : nullptr;
+    const uint4 *br = reinterpret_cast<const uint4 *>(bias);
+    half8 v[kNormMaxVec];
+    float sum = 0.f, ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kNormMaxVec; ++i) {
+        const int c = tid + i * kNormThreads;
+        if (c < nvec) {
+            v[i] = __builtin_bit_cast(half8, xr[c]);
+            if (rr)
+                v[i] = v[i] + __builtin_bit_cast(half8, rr[c]);   // fp16 add, then
+            if (br)
+                v[i] = v[i] + __builtin_bit_cast(half8, br[c]);   // a second fp16 add (:58)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float f = (float)v[i][e];
+                sum += f;
+                ss += f * f;
+            }
+        }
+    }
+    auto block_sum = [&](float a, int slot) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1)
+            a += __shfl_xor(a, off, 64);
+        if ((tid & 63) == 0)
+            red[slot][tid >> 6] = a;
+        __syncthreads();
+        float tot = 0.f;
+#pragma unroll
+        for (int w = 0; w < kNormThreads / 64; ++w)
+            tot += red[slot][w];
+        return tot;
+    };
+    float mean = 0.f, inv;
+    if (beta != nullptr) {
+        mean = block_sum(sum, 0) / (float)N;
+        float var = 0.f;
+#pragma unroll
+        for (int i = 0; i < kNormMaxVec; ++i) {
+            const int c = tid + i * kNormThreads;
+            if (c < nvec) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float d = (float)v[i][e] - mean;
+                    var += d * d;
+                }
+            }
+        }
+        inv = rsqrtf(block_sum(var, 1) / (float)N + eps);
+    } else {
+        inv = rsqrtf(block_sum(ss, 0) / (float)N + eps);
+    }
+    const uint4 *gr = reinterpret_cast<const uint4 *>(gamma);
+    const uint4 *ber = reinterpret_cast<const uint4 *>(beta);
+    uint4 *orow = reinterpret_cast<uint4 *>(out + (size_t)row * N);
+#pragma unroll
+    for (int i = 0; i < kNormMaxVec; ++i) {
+        const int c = tid + i * kNormThreads;
+        if (c < nvec) {
+            const half8 g = __builtin_bit_cast(half8, gr[c]);
+            half8 o;
+            if (beta != nullptr) {
+                const half8 be = __builtin_bit_cast(half8, ber[c]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    o[e] = (_Float16)(((float)v[i][e] - mean) * inv * (float)g[e] + (float)be[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    o[e] = (_Float16)((float)v[i][e] * inv * (float)g[e]);
+            }
+            orow[c] = __builtin_bit_cast(uint4, o);
+        }
+    }
+}
+
+// out[m][:] += bias[:] in fp16 (add_bias, csrc/core/add_bias.cu:5-11)
+__global__ void add_bias_kernel(_Float16 *__restrict__ out, const _Float16 *__restrict__ bias, size_t nvec, int nvec_row)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nvec)
+        return;
+    uint4 *o = reinterpret_cast<uint4 *>(out);
+    const half8 b = __builtin_bit_cast(half8, reinterpret_cast<const uint4 *>(bias)[i % nvec_row]);
+    o[i] = __builtin_bit_cast(uint4, __builtin_bit_cast(half8, o[i]) + b);
+}
+
+// ---------------------------------------------------------------------------
 // Fused-QKV split.  qkv[B][S][3][H][dh] -> q_out[B][H][S][dh] and cache rows
 // k_cache / v_cache[b][h][t0 + s][:].  With rope, pairs (i, i + dh/2) of q and
 // k are rotated by angle pos / 10000^(2i/dh) in fp32 (csrc/core/common.cuh:
@@ -212,6 +318,55 @@ extern "C" int eet_rmsnorm(const void *x, const void *gamma, void *out, int M, i
     hipLaunchKernelGGL(rmsnorm_kernel, dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream),
                        static_cast<const _Float16 *>(x), static_cast<const _Float16 *>(gamma),
                        static_cast<_Float16 *>(out), N, eps);
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
+extern "C" int eet_layernorm(const void *x, const void *gamma, const void *beta, void *out, int M, int N, float eps,
+                             void *stream)
+{
+    EET_REQUIRE(x && gamma && beta && out, EET_ERR_INVALID_ARGUMENT, "eet_layernorm: null pointer");
+    EET_REQUIRE(M >= 0 && N > 0, EET_ERR_INVALID_ARGUMENT, "eet_layernorm: bad sizes M=%d N=%d", M, N);
+    EET_REQUIRE(N % 8 == 0 && N <= kNormThreads * kNormMaxVec * 8, EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_layernorm: need N %% 8 == 0 and N <= 16384, got %d", N);
+    if (M == 0)
+        return EET_OK;
+    hipLaunchKernelGGL(add_norm_kernel, dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const _Float16 *>(x), static_cast<const _Float16 *>(nullptr),
+                       static_cast<const _Float16 *>(nullptr), static_cast<const _Float16 *>(gamma),
+                       static_cast<const _Float16 *>(beta), static_cast<_Float16 *>(out), N, eps);
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
+extern "C" int eet_add_bias_residual_norm(void *out, const void *input, const void *bias, const void *gamma,
+                                          const void *beta, int M, int N, float eps, void *stream)
+{
+    EET_REQUIRE(out && input && gamma, EET_ERR_INVALID_ARGUMENT, "eet_add_bias_residual_norm: null pointer");
+    EET_REQUIRE(M >= 0 && N > 0, EET_ERR_INVALID_ARGUMENT, "eet_add_bias_residual_norm: bad sizes M=%d N=%d", M, N);
+    EET_REQUIRE(N % 8 == 0 && N <= kNormThreads * kNormMaxVec * 8, EET_ERR_UNSUPPORTED_SHAPE,
+                "eet_add_bias_residual_norm: need N %% 8 == 0 and N <= 16384, got %d", N);
+    if (M == 0)
+        return EET_OK;
+    hipLaunchKernelGGL(add_norm_kernel, dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const _Float16 *>(out), static_cast<const _Float16 *>(input),
+                       static_cast<const _Float16 *>(bias), static_cast<const _Float16 *>(gamma),
+                       static_cast<const _Float16 *>(beta), static_cast<_Float16 *>(out), N, eps);
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
+extern "C" int eet_add_bias(void *out, const void *bias, int M, int N, void *stream)
+{
+    EET_REQUIRE(out && bias, EET_ERR_INVALID_ARGUMENT, "eet_add_bias: null pointer");
+    EET_REQUIRE(M >= 0 && N > 0, EET_ERR_INVALID_ARGUMENT, "eet_add_bias: bad sizes M=%d N=%d", M, N);
+    EET_REQUIRE(N % 8 == 0, EET_ERR_UNSUPPORTED_SHAPE, "eet_add_bias: need N %% 8 == 0, got %d", N);
+    const size_t nvec = (size_t)M * N / 8;
+    if (nvec == 0)
+        return EET_OK;
+    hipLaunchKernelGGL(add_bias_kernel, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<_Float16 *>(out),
+                       static_cast<const _Float16 *>(bias), nvec, N / 8);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }

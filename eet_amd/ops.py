@@ -278,16 +278,30 @@ class _MmhaInt8:
     """Shared body of LlamaMmha (rotary) and BaichuanMmha (ALiBi)."""
 
     _rope = True
+    _bias_branch = False
     _name = "LlamaMmha"
 
     def __init__(self, desc, QKV_weights, QKV_scale, Q_bias, K_bias, V_bias, Output_weights, Output_scale,
                  Output_bias, layernorm_weights, layernorm_bias):
         _require_int8_fp16(desc, self._name)
-        for nm, b in (("Q_bias", Q_bias), ("K_bias", K_bias), ("V_bias", V_bias), ("Output_bias", Output_bias),
-                      ("layernorm_bias", layernorm_bias)):
-            if b is not None and b.numel() != 0:
-                raise NotImplementedError(f"[EET][ERROR] {self._name}: {nm} is not supported on the int8 path "
-                                          "(LLaMA / Baichuan have none)")
+
+        def given(b):
+            return b is not None and b.numel() != 0
+        # The bias branch: a Q bias switches the op to LayerNorm(gamma, beta) and adds Q / K / V biases to
+        # the fused QKV rows (csrc/op/baichuan_mmha.cpp:45, 224-231, 295-297); the output bias follows
+        # the residual add (:402).
+        self.with_bias = given(Q_bias)
+        if self.with_bias and not self._bias_branch:
+            # for fp16 the reference's rotary split prints "Not support add bias for half" and launches
+            # nothing (csrc/core/self_add_bias.cu:476-480): there is no behaviour to reproduce
+            raise NotImplementedError(f"[EET][ERROR] {self._name}: Q / K / V biases are not supported with fp16 "
+                                      "(the reference's rotary split refuses them for half as well)")
+        if not self.with_bias and (given(K_bias) or given(V_bias) or given(layernorm_bias)):
+            raise RuntimeError(f"[EET][ERROR] {self._name}: K_bias, V_bias and layernorm_bias take effect only "
+                               "together with Q_bias (the reference selects the bias branch by Q_bias alone)")
+        if self.with_bias and not (given(K_bias) and given(V_bias) and given(layernorm_bias)):
+            raise RuntimeError(f"[EET][ERROR] {self._name}: with Q_bias the op also reads K_bias, V_bias and "
+                               "layernorm_bias; all must be given")
         self.desc = desc
         H = desc.head_num
         if desc.d_kv == 0:
@@ -313,6 +327,17 @@ class _MmhaInt8:
         self.step = 1
         self.first_batch = 0
         self.rope_table = _rope_table(self.t_cap, self.dh, dev) if self._rope else None
+        self.qkv_bias = self.beta = self.o_bias = None
+        if self.with_bias:
+            for nm, b in (("Q_bias", Q_bias), ("K_bias", K_bias), ("V_bias", V_bias)):
+                _check_vec(nm, b, self.inner)
+            _check_vec("layernorm_bias", layernorm_bias, hidden)
+            self.qkv_bias = torch.cat((Q_bias.reshape(-1), K_bias.reshape(-1), V_bias.reshape(-1))).contiguous()
+            self.beta = layernorm_bias
+        if given(Output_bias):
+            _check_vec("Output_bias", Output_bias, hidden)
+            self.o_bias = Output_bias
+        self.biased = self.with_bias or self.o_bias is not None
 
     def forward(self, input, pre_padding_len, reorder_state, pre_layernorm, add_residual, first_pass,
                 relative_attention_bias=_EMPTY):
@@ -382,7 +407,9 @@ class _MmhaInt8:
         qbuf = workspaces.get("q_buf", desc.batch_size * max(desc.max_seq_len, 1) * self.inner, f16, dev)
         cbuf = workspaces.get("context_buf", desc.batch_size * max(desc.max_seq_len, 1) * self.inner, f16, dev)
         out = workspaces.get("self_mask_attn_cache", desc.batch_size * max(desc.max_seq_len, 1) * hidden, f16, dev)
-        if not first_pass and M <= RMS_FUSE_MAX_M:
+        if self.biased and replay_state is not None:
+            raise NotImplementedError(f"[EET][ERROR] {self._name}: the bias branch has no replayable (HIP graph) form")
+        if not first_pass and M <= RMS_FUSE_MAX_M and not self.biased:
             # the whole incremental call from one library call: RMSnorm + QKV, rotary + append +
             # attention, output projection + residual
             alibi = None
@@ -436,7 +463,14 @@ class _MmhaInt8:
                                          ws.numel() * 4, _stream()), "eet_mmha_int8_decode")
             self._keep = (x, pad, alibi, reorder)  # inputs of kernels still in flight
             return out[: M * hidden].view(B, S, hidden)
-        if M <= RMS_FUSE_MAX_M:
+        if self.with_bias:
+            # LayerNorm, QKV projection, then the three biases on the fused rows (fp16 adds, as
+            # fused_add_QKV_bias makes them: csrc/core/self_add_bias.cu:352-354)
+            check(L.eet_layernorm(x.data_ptr(), self.gamma.data_ptr(), self.beta.data_ptr(), xn.data_ptr(), M, hidden,
+                                  desc.layernorm_eps, _stream()), "eet_layernorm")
+            _gemm(xn, self.qkv_w, self.qkv_s, qkv, M, 3 * self.inner, hidden)
+            check(L.eet_add_bias(qkv.data_ptr(), self.qkv_bias.data_ptr(), M, 3 * self.inner, _stream()), "eet_add_bias")
+        elif M <= RMS_FUSE_MAX_M:
             # RMSnorm folded into the GEMM's activation load
             _gemm(x, self.qkv_w, self.qkv_s, qkv, M, 3 * self.inner, hidden, EPI_NONE, None, self.gamma,
                   desc.layernorm_eps)
@@ -476,6 +510,8 @@ class _MmhaInt8:
                   "eet_mmha_decode")
         # output projection with the residual add (csrc/op/llama_mmha.cpp:428-462) in its epilogue
         _gemm(cbuf, self.o_w, self.o_s, out, M, hidden, self.inner, EPI_RESIDUAL, x)
+        if self.o_bias is not None:     # (out + input) + bias, csrc/core/add_bias.cu:13-20
+            check(L.eet_add_bias(out.data_ptr(), self.o_bias.data_ptr(), M, hidden, _stream()), "eet_add_bias")
         self._keep = (x, pad, alibi, reorder)  # inputs of kernels still in flight
         return out[: M * hidden].view(B, S, hidden)
 
@@ -483,6 +519,7 @@ class _MmhaInt8:
 class LlamaMmha(_MmhaInt8):
     """csrc/op/llama_mmha.cpp:14-266."""
     _rope = True
+    _bias_branch = False
     _name = "LlamaMmha"
 
 
@@ -490,6 +527,7 @@ class BaichuanMmha(_MmhaInt8):
     """csrc/op/baichuan_mmha.cpp:81-216: no rotary; an ALiBi tensor is passed in
     ([H, S, S] for the prompt, [H, 1, step] per decode step)."""
     _rope = False
+    _bias_branch = True
     _name = "BaichuanMmha"
 
 
@@ -507,10 +545,8 @@ class GatedFeedForwardNetworkInt8:
             # the reference prints "unsupported activation" and goes on (gated_ffn_int8.cpp:57-61)
             raise NotImplementedError(f"[EET][ERROR] GatedFeedForwardNetworkInt8: activation "
                                       f"'{desc.activation_fn}' is not implemented (silu only)")
-        for nm, b in (("Intermediate_0_bias", Intermediate_0_bias), ("Intermediate_1_bias", Intermediate_1_bias),
-                      ("Output_bias", Output_bias), ("layernorm_bias", layernorm_bias)):
-            if b is not None and b.numel() != 0:
-                raise NotImplementedError(f"[EET][ERROR] GatedFeedForwardNetworkInt8: {nm} is not supported")
+        # Intermediate_0_bias / Intermediate_1_bias are accepted and never used, exactly as in the reference:
+        # its forward passes no bias to fc1 / fc2 and gated_act takes none (gated_ffn_int8.cpp:98-132, 168-179).
         self.desc = desc
         hidden = desc.hidden_units
         self.d_ff = desc.d_ff if desc.d_ff != 0 else 4 * hidden  # gated_ffn_int8.cpp:62-68
@@ -523,6 +559,13 @@ class GatedFeedForwardNetworkInt8:
         _check_vec("Output_scale", Output_scale, hidden)
         _check_vec("layernorm_weights", layernorm_weights, hidden)
         self.w2, self.s2, self.gamma = Output_weights, Output_scale, layernorm_weights
+        self.beta = self.o_bias = None
+        if layernorm_bias is not None and layernorm_bias.numel() != 0:    # LayerNorm instead of RMSnorm (:139-146)
+            _check_vec("layernorm_bias", layernorm_bias, hidden)
+            self.beta = layernorm_bias
+        if Output_bias is not None and Output_bias.numel() != 0:
+            _check_vec("Output_bias", Output_bias, hidden)
+            self.o_bias = Output_bias
         self.cache_name = ffn_cache_name
         # gate and up merged tile by tile so that one launch computes both and applies SwiGLU;
         # the op keeps only the merged copy (the caller's separate tensors can be freed)
@@ -538,8 +581,10 @@ class GatedFeedForwardNetworkInt8:
         if input.dtype != torch.float16 or input.dim() != 3 or input.shape[2] != desc.hidden_units:
             raise RuntimeError(f"[EET][ERROR] GatedFeedForwardNetworkInt8: input must be fp16 [B, S, "
                                f"{desc.hidden_units}], got {input.dtype} {tuple(input.shape)}")
-        if add_residual and not pre_layernorm:
-            raise NotImplementedError("[EET][ERROR] GatedFeedForwardNetworkInt8: post-layernorm mode is not implemented")
+        post_ln = add_residual and not pre_layernorm
+        if post_ln and self.o_bias is not None and self.beta is None:
+            raise RuntimeError("[EET][ERROR] GatedFeedForwardNetworkInt8: the post-layernorm tail with an output bias is "
+                               "a LayerNorm and needs layernorm_bias (gated_ffn_int8.cpp:335-342)")
         x = input.contiguous()
         B, S, hidden = x.shape
         if B > desc.batch_size or S > max(desc.max_seq_len, 1):
@@ -550,6 +595,8 @@ class GatedFeedForwardNetworkInt8:
         xn = workspaces.get("layernorm_tensor", cap * hidden, f16, dev)
         act = workspaces.get("ffn_inner_act", cap * self.d_ff, f16, dev)
         out = workspaces.get(self.cache_name, cap * hidden, f16, dev)
+        if post_ln or self.beta is not None or self.o_bias is not None:
+            return self._forward_general(x, xn, act, out, M, hidden, post_ln, add_residual)
         # fc1, fc2 and gated_act (gated_ffn_int8.cpp:253-301, 168-179) in one launch; at decode
         # sizes the RMSnorm (:112) rides in the same launch and fc3 follows from the same library call
         if M <= RMS_FUSE_MAX_M and launch_timer is not None:
@@ -579,15 +626,44 @@ class GatedFeedForwardNetworkInt8:
         return out[: M * hidden].view(B, S, hidden)
 
 
+    def _forward_general(self, x, xn, act, out, M, hidden, post_ln, add_residual):
+        """The branches LLaMA / Baichuan never take: LayerNorm in front (layernorm_bias given), an output bias,
+        and the post-layernorm tail.  Unfused: norm kernel, gate|up + SwiGLU, down, then the tail."""
+        desc, L, B, S = self.desc, lib(), x.shape[0], x.shape[1]
+        if self.beta is not None:
+            check(L.eet_layernorm(x.data_ptr(), self.gamma.data_ptr(), self.beta.data_ptr(), xn.data_ptr(), M, hidden,
+                                  desc.layernorm_eps, _stream()), "eet_layernorm")
+        else:
+            _rmsnorm(x, self.gamma, xn, M, hidden, desc.layernorm_eps)     # applied in both modes (:112)
+        _gemm(xn, self.w01, self.s01, act, M, 2 * self.d_ff, hidden, EPI_SWIGLU)
+        if post_ln:
+            # add_bias + add_residual + layer_norm (:335-342): LayerNorm with a bias, RMSnorm without
+            _gemm(act, self.w2, self.s2, out, M, hidden, self.d_ff)
+            check(L.eet_add_bias_residual_norm(out.data_ptr(), x.data_ptr(), _ptr(self.o_bias), self.gamma.data_ptr(),
+                                               self.beta.data_ptr() if self.o_bias is not None else None, M, hidden,
+                                               desc.layernorm_eps, _stream()), "eet_add_bias_residual_norm")
+        else:
+            if add_residual:
+                _gemm(act, self.w2, self.s2, out, M, hidden, self.d_ff, EPI_RESIDUAL, x)
+            else:
+                _gemm(act, self.w2, self.s2, out, M, hidden, self.d_ff)
+            if self.o_bias is not None:
+                check(L.eet_add_bias(out.data_ptr(), self.o_bias.data_ptr(), M, hidden, _stream()), "eet_add_bias")
+        self._keep = x
+        return out[: M * hidden].view(B, S, hidden)
+
+
 class LayerNorm:
-    """csrc/op/layer_norm.cpp:8-33: RMSnorm when beta is empty."""
+    """csrc/op/layer_norm.cpp:8-33: LayerNorm(gamma, beta), RMSnorm when beta is empty."""
 
     def __init__(self, desc, gamma, beta):
         if desc.dtype != torch.float16:
             raise NotImplementedError("[EET][ERROR] LayerNorm: fp16 only")
-        if beta is not None and beta.numel() != 0:
-            raise NotImplementedError("[EET][ERROR] LayerNorm: only the RMSnorm form (empty beta) is implemented")
         _check_vec("gamma", gamma, desc.hidden_units)
+        self.beta = None
+        if beta is not None and beta.numel() != 0:
+            _check_vec("beta", beta, desc.hidden_units)
+            self.beta = beta
         self.desc, self.gamma = desc, gamma
         self.output = torch.zeros(desc.batch_size, max(desc.max_seq_len, 1), desc.hidden_units,
                                   dtype=torch.float16, device=gamma.device)
@@ -600,7 +676,11 @@ class LayerNorm:
         B, S, hidden = x.shape
         if B * S > self.output.shape[0] * self.output.shape[1]:
             raise RuntimeError("[EET][ERROR] LayerNorm: input larger than batch_size * max_seq_len")
-        _rmsnorm(x, self.gamma, self.output, B * S, hidden, desc.layernorm_eps)
+        if self.beta is not None:
+            check(lib().eet_layernorm(x.data_ptr(), self.gamma.data_ptr(), self.beta.data_ptr(), self.output.data_ptr(),
+                                      B * S, hidden, desc.layernorm_eps, _stream()), "eet_layernorm")
+        else:
+            _rmsnorm(x, self.gamma, self.output, B * S, hidden, desc.layernorm_eps)
         self._keep = x
         return self.output.view(-1)[: B * S * hidden].view(B, S, hidden)
 

@@ -249,6 +249,26 @@ int eet_rope_table(float *table, int T, int dh, void *stream);
 int eet_rmsnorm(const void *x, const void *gamma, void *out, int M, int N, float eps,
                 void *stream);
 
+/* out[M][N] = (x - mean(x)) * rsqrt(var(x) + eps) * gamma + beta: the LayerNorm the
+ * ops use instead of RMSnorm when they are given biases.  fp32 statistics (mean,
+ * then the variance of the centred values), one rounding.  Replaces layernorm
+ * (csrc/core/layer_norm.cu:533-578, kernel :384-446). */
+int eet_layernorm(const void *x, const void *gamma, const void *beta, void *out, int M, int N,
+                  float eps, void *stream);
+
+/* In place: out[M][N] = norm((out + input) [+ bias]) with the two adds in fp16 as the
+ * reference makes them; norm is LayerNorm(gamma, beta) when beta is given and
+ * RMSnorm(gamma) when beta is NULL; bias may be NULL.  The post-layernorm tail of
+ * the feed-forward op.  Replaces add_bias_input_layernorm_kernel
+ * (csrc/core/layer_norm.cu:627-668; kernels :39-80 and :103-131) without its
+ * N <= 2048 limit. */
+int eet_add_bias_residual_norm(void *out, const void *input, const void *bias, const void *gamma,
+                               const void *beta, int M, int N, float eps, void *stream);
+
+/* out[M][N] += bias[N] (fp16 add).  Replaces add_bias_kernel
+ * (csrc/core/add_bias.cu:30-49) and the bias half of add_bias_input_kernel (:51-73). */
+int eet_add_bias(void *out, const void *bias, int M, int N, void *stream);
+
 /* Split a fused qkv[B][S][3][H][dh] row.  With rope != 0, q and k are rotated
  * NeoX-style (pairs i, i + dh/2) at position s (time_step < 0) or time_step.
  *   q_out  [B][H][S][dh]

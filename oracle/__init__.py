@@ -18,6 +18,9 @@ checkout).  How each function is pinned:
   dequant_matmul         textbook fp32 matmul; identity / one-hot special cases
   rmsnorm, swiglu, rope  closed forms, norm preservation, pos=0 identity,
                          equality with the rotate_half formulation
+  layernorm, add_bias,   float64 textbook LayerNorm (zero mean / unit variance with
+  add_bias_residual_norm gamma = 1, beta = 0; shift and scale invariance), the two fp16 adds
+                         brute-forced element by element, RMSnorm form without a bias
   decode_attention       step=1 => v/(1+1e-6), uniform keys => mean(V),
                          brute-force softmax, padded prefix has zero weight
   alibi_slopes / mask    closed form for n=40 and powers of two

@@ -79,6 +79,33 @@ def qkv_split(qkv, B, S, H, dh, rope, time_step=-1):
     return q, k, v
 
 
+def layernorm(x, gamma, beta, eps):
+    """(x - mean) * rsqrt(var + eps) * gamma + beta, fp32 statistics (variance of the centred
+    values over n), fp16 out.  csrc/core/layer_norm.cu:384-446 (decoder_norm1_kernel_opt, half)."""
+    xf = x.astype(F32)
+    mean = np.mean(xf, axis=-1, keepdims=True, dtype=F32)
+    d = xf - mean
+    var = np.mean(d * d, axis=-1, keepdims=True, dtype=F32)
+    inv = (F32(1.0) / np.sqrt(var + F32(eps))).astype(F32)
+    return (d * inv * gamma.astype(F32) + beta.astype(F32)).astype(F16)
+
+
+def add_bias(out, bias):
+    """out + bias in fp16.  csrc/core/add_bias.cu:5-11."""
+    return (out.astype(F16) + bias.astype(F16)[None, :]).astype(F16)
+
+
+def add_bias_residual_norm(out, inp, bias, gamma, beta, eps):
+    """Post-layernorm tail of the feed-forward op: y = (out + inp) [+ bias] with fp16 adds, then
+    LayerNorm(gamma, beta) when a bias is given, RMSnorm(gamma) otherwise.
+    csrc/core/layer_norm.cu:39-80 (add_bias_input_layernorm, half), :103-131 (add_input_RMSnorm,
+    half); selected by bias != nullptr at :650-666."""
+    y = residual_add(out, inp)
+    if bias is not None:
+        return layernorm(add_bias(y, bias), gamma, beta, eps)
+    return rmsnorm(y, gamma, eps)
+
+
 def swiglu(gate, up):
     """up * gate / (1 + exp(-gate)).  csrc/core/activation_kernel.cu:106-124.
     (The reference does the multiply / divide in half2; here once in fp32.)"""
@@ -214,9 +241,15 @@ class OracleAttention:
     csrc/op/baichuan_mmha.cpp:81-216.  Weights are the *unprocessed* int8
     [K, N] matrices plus fp16 scales."""
 
-    def __init__(self, B, H, dh, cap, qkv_q, qkv_s, o_q, o_s, gamma, eps, rope=True):
+    def __init__(self, B, H, dh, cap, qkv_q, qkv_s, o_q, o_s, gamma, eps, rope=True, qkv_bias=None, o_bias=None,
+                 beta=None):
+        """qkv_bias [3 * H * dh] (q | k | v), beta: the bias branch of BaichuanMmha -- with a Q bias the op
+        normalises with LayerNorm(gamma, beta) instead of RMSnorm (csrc/op/baichuan_mmha.cpp:45, 224-231)
+        and adds the biases to the fused QKV rows in fp16 (:295-297, csrc/core/self_add_bias.cu:352-354);
+        o_bias is added after the residual (:402, csrc/core/add_bias.cu:13-20)."""
         self.H, self.dh, self.rope, self.eps = H, dh, rope, eps
         self.qkv_q, self.qkv_s, self.o_q, self.o_s, self.gamma = qkv_q, qkv_s, o_q, o_s, gamma
+        self.qkv_bias, self.o_bias, self.beta = qkv_bias, o_bias, beta
         self.k_cache = np.zeros((B, H, cap, dh), F16)
         self.v_cache = np.zeros((B, H, cap, dh), F16)
         self.step = 1
@@ -226,8 +259,12 @@ class OracleAttention:
         H, dh = self.H, self.dh
         if reorder is not None and not first_pass:
             reorder_cache(self.k_cache, self.v_cache, reorder, self.step)
-        xn = rmsnorm(x.reshape(B * S, hidden), self.gamma, self.eps)
-        qkv = dequant_matmul(xn, self.qkv_q, self.qkv_s)
+        if self.qkv_bias is not None:
+            xn = layernorm(x.reshape(B * S, hidden), self.gamma, self.beta, self.eps)
+            qkv = add_bias(dequant_matmul(xn, self.qkv_q, self.qkv_s), self.qkv_bias)
+        else:
+            xn = rmsnorm(x.reshape(B * S, hidden), self.gamma, self.eps)
+            qkv = dequant_matmul(xn, self.qkv_q, self.qkv_s)
         if first_pass:
             q, k, v = qkv_split(qkv, B, S, H, dh, self.rope, -1)
             self.k_cache[:B, :, :S] = k
@@ -240,24 +277,38 @@ class OracleAttention:
             q, k, v = qkv_split(qkv, B, 1, H, dh, self.rope, self.step - 1)
             ctx = decode_attention(q[:, :, 0], k[:, :, 0], v[:, :, 0], self.k_cache[:B], self.v_cache[:B],
                                    self.step, pad, alibi)
-        out = dequant_matmul(ctx.reshape(B * S, H * dh), self.o_q, self.o_s)
-        return residual_add(out, x.reshape(B * S, hidden)).reshape(B, S, hidden)
+        out = residual_add(dequant_matmul(ctx.reshape(B * S, H * dh), self.o_q, self.o_s), x.reshape(B * S, hidden))
+        if self.o_bias is not None:
+            out = add_bias(out, self.o_bias)
+        return out.reshape(B, S, hidden)
 
 
 class OracleFFN:
     """GatedFeedForwardNetworkInt8 restated.  csrc/op/gated_ffn_int8.cpp:98-132."""
 
-    def __init__(self, g_q, g_s, u_q, u_s, d_q, d_s, gamma, eps):
+    def __init__(self, g_q, g_s, u_q, u_s, d_q, d_s, gamma, eps, beta=None, o_bias=None):
+        """beta: with a layernorm bias the op normalises with LayerNorm (gated_ffn_int8.cpp:139-146);
+        o_bias: the output bias (:328-357).  The two intermediate biases the constructor takes are never
+        read by the reference's forward (:98-132), so they have no place here."""
         self.g_q, self.g_s, self.u_q, self.u_s, self.d_q, self.d_s = g_q, g_s, u_q, u_s, d_q, d_s
-        self.gamma, self.eps = gamma, eps
+        self.gamma, self.eps, self.beta, self.o_bias = gamma, eps, beta, o_bias
 
-    def forward(self, x):
+    def forward(self, x, pre_layernorm=True, add_residual=True):
         B, S, hidden = x.shape
         x2 = x.reshape(B * S, hidden)
-        xn = rmsnorm(x2, self.gamma, self.eps)
+        # the norm in front is applied in both modes (:112)
+        xn = layernorm(x2, self.gamma, self.beta, self.eps) if self.beta is not None else rmsnorm(x2, self.gamma, self.eps)
         act = swiglu(dequant_matmul(xn, self.g_q, self.g_s), dequant_matmul(xn, self.u_q, self.u_s))
         out = dequant_matmul(act, self.d_q, self.d_s)
-        return residual_add(out, x2).reshape(B, S, hidden)
+        if add_residual and not pre_layernorm:       # post-layernorm mode (:335-342)
+            out = add_bias_residual_norm(out, x2, self.o_bias, self.gamma, self.beta, self.eps)
+        elif add_residual:                           # (:343-347)
+            out = residual_add(out, x2)
+            if self.o_bias is not None:
+                out = add_bias(out, self.o_bias)
+        elif self.o_bias is not None:                # (:349-355)
+            out = add_bias(out, self.o_bias)
+        return out.reshape(B, S, hidden)
 
 
 class OracleDecoder:

@@ -240,3 +240,59 @@ def test_greedy_tokens_match_hf_formulation():
             if top2[b, 1] - top2[b, 0] > 0.05:        # margin above the fp16 noise of the oracle
                 assert toks[b, t] == nxt[b]
         seq = np.concatenate([seq, toks[:, t:t + 1]], 1)     # follow the oracle's tokens
+
+
+def test_bias_branch_one_token_closed_form():
+    """The bias branch of the attention op on a one-token prompt, where attention is the identity on v:
+    out = x + Wo . ((LN(x) . Wv + bv) / (1 + 1e-6)) + bo, with LayerNorm(gamma, beta) in front.  And the
+    feed-forward op in its three tails against the float64 formulas."""
+    rng = np.random.default_rng(21)
+    hidden, heads, d_ff = 128, 4, 192
+
+    def linear(i, o):
+        q, s = Q.quantize_ref128(np.ascontiguousarray((rng.standard_normal((i, o)) * 0.08).astype(np.float16)))
+        return q, s, q.astype(np.float64) * s.astype(np.float64)[None, :]
+    qkv_q, qkv_s, wqkv = linear(hidden, 3 * hidden)
+    o_q, o_s, wo = linear(hidden, hidden)
+    g = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float16)
+    beta = (0.2 * rng.standard_normal(hidden)).astype(np.float16)
+    qkv_b = (0.3 * rng.standard_normal(3 * hidden)).astype(np.float16)
+    o_b = (0.3 * rng.standard_normal(hidden)).astype(np.float16)
+    attn = O.OracleAttention(2, heads, hidden // heads, 8, qkv_q, qkv_s, o_q, o_s, g, EPS, rope=False,
+                             qkv_bias=qkv_b, o_bias=o_b, beta=beta)
+    x = (rng.standard_normal((2, 1, hidden)) + 0.5).astype(np.float16)
+
+    def ln(v):
+        v = v.astype(np.float64)
+        return (v - v.mean(-1, keepdims=True)) / np.sqrt(v.var(-1, keepdims=True) + EPS) * g.astype(np.float64) \
+            + beta.astype(np.float64)
+    v = ln(x) @ wqkv[:, 2 * hidden:] + qkv_b[2 * hidden:].astype(np.float64)
+    want = x.astype(np.float64) + (v / (1 + 1e-6)) @ wo + o_b.astype(np.float64)
+    assert max_rel(attn.forward(x, None, True), want) < 5e-3
+    # the new token's k row in the cache carries its bias
+    k = (ln(x) @ wqkv[:, hidden:2 * hidden] + qkv_b[hidden:2 * hidden].astype(np.float64)).reshape(2, heads, -1)
+    assert np.abs(attn.k_cache[:, :, 0].astype(np.float64) - k).max() < 6e-3
+    # without the bias terms the same formula must NOT match (the comparison sees a dropped bias)
+    assert max_rel(attn.forward(x, None, True), x.astype(np.float64) + ((ln(x) @ wqkv[:, 2 * hidden:]) / (1 + 1e-6)) @ wo) > 0.05
+
+    g_q, g_s, wg = linear(hidden, d_ff)
+    u_q, u_s, wu = linear(hidden, d_ff)
+    d_q, d_s, wd = linear(d_ff, hidden)
+    x2 = (rng.standard_normal((2, 3, hidden)) + 0.5).astype(np.float16)
+
+    def ffn_core(norm):
+        xn = norm(x2)
+        gate, up = xn @ wg, xn @ wu
+        return (up * gate / (1 + np.exp(-gate))) @ wd
+
+    def rms(v):
+        v = v.astype(np.float64)
+        return v / np.sqrt((v * v).mean(-1, keepdims=True) + EPS) * g.astype(np.float64)
+    x64 = x2.astype(np.float64)
+    ffn = O.OracleFFN(g_q, g_s, u_q, u_s, d_q, d_s, g, EPS, beta=beta, o_bias=o_b)
+    assert max_rel(ffn.forward(x2, True, True), x64 + ffn_core(ln) + o_b.astype(np.float64)) < 1e-2
+    assert max_rel(ffn.forward(x2, True, False), ffn_core(ln) + o_b.astype(np.float64)) < 1e-2
+    assert max_rel(ffn.forward(x2, False, True), ln(x64 + ffn_core(ln) + o_b.astype(np.float64))) < 1e-2
+    plain = O.OracleFFN(g_q, g_s, u_q, u_s, d_q, d_s, g, EPS)
+    assert max_rel(plain.forward(x2, False, True), rms(x64 + ffn_core(rms))) < 1e-2      # RMSnorm tail without a bias
+    assert max_rel(plain.forward(x2, True, False), ffn_core(rms)) < 1e-2

@@ -210,3 +210,45 @@ def test_reorder_cache_gather():
     O.reorder_cache(k, v, perm, T)
     O.reorder_cache(k, v, inv, T)
     assert np.array_equal(k, k0) and np.array_equal(v, v0)
+
+
+def test_layernorm_closed_forms():
+    """LayerNorm against the float64 textbook form; zero mean and unit variance out with gamma = 1, beta = 0;
+    invariance under a shift and a scale of the input; beta passes straight through a constant row."""
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal((5, 256)) * 1.7 + 0.8).astype(np.float16)
+    g = (1 + 0.1 * rng.standard_normal(256)).astype(np.float16)
+    b = (0.2 * rng.standard_normal(256)).astype(np.float16)
+    x64 = x.astype(np.float64)
+    mu, var = x64.mean(-1, keepdims=True), x64.var(-1, keepdims=True)       # population variance
+    want = (x64 - mu) / np.sqrt(var + 1e-5) * g.astype(np.float64) + b.astype(np.float64)
+    assert np.abs(O.layernorm(x, g, b, 1e-5).astype(np.float64) - want).max() < 3e-3
+    one, zero = np.ones(256, np.float16), np.zeros(256, np.float16)
+    y = O.layernorm(x, one, zero, 1e-6).astype(np.float64)
+    assert np.abs(y.mean(-1)).max() < 2e-3 and np.allclose((y * y).mean(-1), 1.0, rtol=3e-3)
+    y2 = O.layernorm((x.astype(np.float32) * 2 + 3).astype(np.float16), one, zero, 1e-12).astype(np.float32)
+    assert np.abs(y2 - O.layernorm(x, one, zero, 1e-12).astype(np.float32)).max() < 6e-3
+    const = np.full((2, 256), 4.0, np.float16)       # variance 0: only beta is left
+    assert np.array_equal(O.layernorm(const, g, b, 1e-6), np.broadcast_to(b, (2, 256)))
+    # a dropped mean (RMSnorm in its place) is seen: the input has mean 0.8
+    assert np.abs(O.rmsnorm(x, g, 1e-5).astype(np.float64) + b.astype(np.float64) - want).max() > 0.1
+
+
+def test_bias_and_post_layernorm_tail():
+    rng = np.random.default_rng(4)
+    out = rng.standard_normal((3, 64)).astype(np.float16)
+    inp = rng.standard_normal((3, 64)).astype(np.float16)
+    bias = rng.standard_normal(64).astype(np.float16)
+    g = (1 + 0.1 * rng.standard_normal(64)).astype(np.float16)
+    b = (0.3 * rng.standard_normal(64)).astype(np.float16)
+    # the two adds are fp16 adds, one after the other: brute force, element by element
+    yb = np.array([[np.float16(np.float16(out[m, n] + inp[m, n]) + bias[n]) for n in range(64)] for m in range(3)])
+    assert np.array_equal(O.add_bias(O.residual_add(out, inp), bias), yb)
+    y64 = yb.astype(np.float64)
+    want = (y64 - y64.mean(-1, keepdims=True)) / np.sqrt(y64.var(-1, keepdims=True) + 1e-6) * g.astype(np.float64) \
+        + b.astype(np.float64)
+    assert np.abs(O.add_bias_residual_norm(out, inp, bias, g, b, 1e-6).astype(np.float64) - want).max() < 3e-3
+    # without a bias the tail is an RMSnorm of out + inp (beta is not used)
+    y = O.residual_add(out, inp).astype(np.float64)
+    want = y / np.sqrt((y * y).mean(-1, keepdims=True) + 1e-6) * g.astype(np.float64)
+    assert np.abs(O.add_bias_residual_norm(out, inp, None, g, b, 1e-6).astype(np.float64) - want).max() < 3e-3

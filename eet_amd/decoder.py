@@ -189,6 +189,84 @@ class Int8Decoder:
                 logits = self.logits(nxt[:, None], False, attention_mask)
         return torch.stack(out, dim=1)
 
+    # ---- beam search ----------------------------------------------------------------------------
+    @torch.no_grad()
+    def beam_search(self, input_ids, num_beams, max_new_tokens, eos_token_id=None, pad_token_id=0,
+                    length_penalty=1.0):
+        """Beam search over the decoder (pipelines/generation.py:1379-1680 with the stock beam scorer the
+        reference instantiates at :960-975): every prompt is expanded to num_beams rows; each step takes
+        the log-softmax of the last position, adds the running beam scores, keeps the best 2 * num_beams
+        (beam, token) pairs per prompt in score order, turns end-of-sequence candidates among the first
+        num_beams ranks into finished hypotheses (score = sum of log-probabilities / length ** length_penalty,
+        the length counting the prompt) and continues with the first num_beams others.  The beam each
+        continuation came from is handed to the attention ops as reorder_state with the next call
+        (generation.py:1577), which gathers their KV caches (csrc/op/llama_mmha.cpp:248-252).
+        Returns (tokens [B, <= max_new_tokens] padded with pad_token_id, scores [B])."""
+        cfg = self.cfg
+        B, S = input_ids.shape
+        nb = int(num_beams)
+        if nb < 1 or B * nb > cfg.max_batch:
+            raise RuntimeError(f"[EET][ERROR] beam_search: batch {B} x num_beams {nb} exceeds max_batch {cfg.max_batch}")
+        dev = input_ids.device
+        ids = input_ids.repeat_interleave(nb, 0)                                   # [B * nb, S]
+        beam_scores = torch.zeros(B, nb, dtype=torch.float32, device=dev)
+        beam_scores[:, 1:] = -1e9                                                  # only the first copy counts at step 0
+        gen = torch.empty(B * nb, 0, dtype=torch.long, device=dev)
+        finished = [[] for _ in range(B)]                                          # per prompt: (score, tokens)
+        done = [False] * B
+        self.reorder_state = torch.empty(0, dtype=torch.long)
+        try:
+            logits = self.logits(ids, True)
+            for step in range(max_new_tokens):
+                logp = torch.log_softmax(logits[:, -1, :].float(), dim=-1) + beam_scores.view(-1, 1)
+                V = logp.shape[-1]
+                top_s, top_i = torch.topk(logp.view(B, nb * V), 2 * nb, dim=1, largest=True, sorted=True)
+                top_s, src, tok = top_s.cpu(), (top_i // V).cpu(), (top_i % V).cpu()
+                gen_host = gen.cpu()
+                cur_len = S + step                                                 # tokens before this step's
+                nxt_s = torch.zeros(B, nb)
+                nxt_t = torch.full((B, nb), pad_token_id, dtype=torch.long)
+                nxt_b = torch.zeros(B, nb, dtype=torch.long)
+                for b in range(B):
+                    if done[b]:
+                        continue
+                    k = 0
+                    for rank in range(2 * nb):
+                        sc, sb, tk = float(top_s[b, rank]), int(src[b, rank]), int(tok[b, rank])
+                        if eos_token_id is not None and tk == eos_token_id:
+                            if rank < nb:                                          # an end among the best num_beams
+                                finished[b].append((sc / (cur_len ** length_penalty), gen_host[b * nb + sb].clone()))
+                            continue
+                        nxt_s[b, k], nxt_t[b, k], nxt_b[b, k] = sc, tk, sb
+                        k += 1
+                        if k == nb:
+                            break
+                    if len(finished[b]) >= nb:
+                        finished[b] = sorted(finished[b], key=lambda h: -h[0])[:nb]
+                        best_open = float(top_s[b].max()) / ((cur_len + 1) ** length_penalty)
+                        done[b] = finished[b][-1][0] >= best_open
+                beam_scores = nxt_s.to(dev)
+                beam_idx = (torch.arange(B)[:, None] * nb + nxt_b).view(-1).to(dev)
+                gen = torch.cat([gen[beam_idx], nxt_t.view(-1, 1).to(dev)], dim=1)
+                if all(done) or step == max_new_tokens - 1:
+                    break
+                self.reorder_state = beam_idx                                      # the ops gather their caches
+                logits = self.logits(nxt_t.view(-1, 1).to(dev), False)
+        finally:
+            self.reorder_state = torch.empty(0, dtype=torch.long)
+        gen_host, scores_host = gen.cpu(), beam_scores.cpu()
+        out = torch.full((B, max_new_tokens), pad_token_id, dtype=torch.long)
+        best = torch.zeros(B)
+        for b in range(B):
+            hyps = list(finished[b])
+            if not done[b]:                                                        # open beams count as they stand
+                total = S + gen_host.shape[1]
+                hyps += [(float(scores_host[b, k]) / (total ** length_penalty), gen_host[b * nb + k]) for k in range(nb)]
+            sc, toks = max(hyps, key=lambda h: h[0])
+            out[b, : toks.numel()] = toks
+            best[b] = sc
+        return out, best
+
     # ---- the incremental step as a HIP graph ---------------------------------------------------
     def _shift_host_steps(self, by):
         for attn, _ in self.layers:

@@ -320,7 +320,7 @@ class OracleDecoder:
         self.embed, self.layers, self.final_gamma, self.lm_head, self.eps = embed, layers, final_gamma, lm_head, eps
         self.alibi, self.n_head, self.past = alibi, n_head, 0
 
-    def step(self, ids, first_pass, pad=None):
+    def step(self, ids, first_pass, pad=None, reorder=None):
         x = self.embed[ids]
         B, S, _ = x.shape
         bias = None
@@ -328,7 +328,7 @@ class OracleDecoder:
             self.past = S if first_pass else self.past + 1
             bias = alibi_mask(self.n_head, self.past) if first_pass else alibi_bias(self.n_head, self.past)
         for attn, ffn in self.layers:
-            x = ffn.forward(attn.forward(x, pad, first_pass, bias))
+            x = ffn.forward(attn.forward(x, pad, first_pass, bias, reorder))
         x = rmsnorm(x, self.final_gamma, self.eps)
         return (x[:, -1].astype(F32) @ self.lm_head.astype(F32).T)
 
@@ -340,3 +340,70 @@ class OracleDecoder:
             out.append(nxt)
             logits = self.step(nxt[:, None], False, pad)
         return np.stack(out, axis=1)
+
+
+    def beam_search(self, ids, num_beams, n_new, eos=None, pad_token=0, length_penalty=1.0):
+        """python/eet/pipelines/generation.py:1379-1680 with the beam scorer of :960-975, restated for the
+        checker: rows [b * num_beams + k]; scores accumulate log-softmax values; 2 * num_beams candidates per
+        prompt in score order; an end-of-sequence candidate ranked inside the first num_beams closes a
+        hypothesis scored sum / length ** length_penalty (length with the prompt); the source beams are
+        handed to the layers as the cache reorder of the next step (:1577)."""
+        return beam_search(lambda x, first, reorder: self.step(x, first, None, reorder), ids, num_beams, n_new, eos,
+                           pad_token, length_penalty)
+
+
+def beam_search(step_fn, ids, nb, n_new, eos=None, pad_token=0, length_penalty=1.0):
+    """The search itself over any next-token function step_fn(ids [rows, S], first_pass, reorder) -> logits
+    [rows, V] (so that tests can pin it with an exhaustive search over a small vocabulary)."""
+    B, S = ids.shape
+    rows = np.repeat(ids, nb, axis=0)
+    score = np.zeros((B, nb), np.float64)
+    score[:, 1:] = -1e9
+    gen = np.zeros((B * nb, 0), np.int64)
+    closed = [[] for _ in range(B)]
+    done = np.zeros(B, bool)
+    logits = step_fn(rows, True, None)
+    for t in range(n_new):
+        z = logits.astype(np.float64)
+        z = z - z.max(-1, keepdims=True)
+        logp = z - np.log(np.exp(z).sum(-1, keepdims=True)) + score.reshape(-1, 1)
+        V = logp.shape[-1]
+        flat = logp.reshape(B, nb * V)
+        order = np.argsort(-flat, axis=1, kind="stable")[:, : 2 * nb]
+        length = S + t
+        new_score = np.zeros((B, nb))
+        new_tok = np.full((B, nb), pad_token, np.int64)
+        new_src = np.zeros((B, nb), np.int64)
+        for b in range(B):
+            if done[b]:
+                continue
+            kept = 0
+            for rank, cand in enumerate(order[b]):
+                beam, tok, sc = cand // V, cand % V, flat[b, cand]
+                if eos is not None and tok == eos:
+                    if rank < nb:
+                        closed[b].append((sc / length ** length_penalty, gen[b * nb + beam].copy()))
+                    continue
+                new_score[b, kept], new_tok[b, kept], new_src[b, kept] = sc, tok, beam
+                kept += 1
+                if kept == nb:
+                    break
+            if len(closed[b]) >= nb:
+                closed[b] = sorted(closed[b], key=lambda h: -h[0])[:nb]
+                done[b] = closed[b][-1][0] >= flat[b, order[b, 0]] / (length + 1) ** length_penalty
+        score = new_score
+        src_rows = (np.arange(B)[:, None] * nb + new_src).reshape(-1)
+        gen = np.concatenate([gen[src_rows], new_tok.reshape(-1, 1)], axis=1)
+        if done.all() or t == n_new - 1:
+            break
+        logits = step_fn(new_tok.reshape(-1, 1), False, src_rows)
+    out = np.full((B, n_new), pad_token, np.int64)
+    best = np.zeros(B)
+    for b in range(B):
+        hyps = list(closed[b])
+        if not done[b]:
+            hyps += [(score[b, k] / (S + gen.shape[1]) ** length_penalty, gen[b * nb + k]) for k in range(nb)]
+        sc, toks = max(hyps, key=lambda h: h[0])
+        out[b, : len(toks)] = toks
+        best[b] = sc
+    return out, best

@@ -225,6 +225,28 @@ def test_beam_search_reorder(gpu, alibi):
                      D.alibi_mask(cfg.heads, step + 1)[:, -1:, :].contiguous().to(gpu) if alibi else torch.empty(0))
 
 
+@pytest.mark.parametrize("alibi,eos", [(False, None), (True, None), (False, 7)])
+def test_beam_search_driver(gpu, alibi, eos):
+    """Int8Decoder.beam_search (the caller of reorder_state: generation.py:1564-1580) against the oracle
+    decoder's beam search: the same sequences, scores within the logits' tolerance; one beam is greedy."""
+    cfg = D.DecoderConfig(num_layers=2, hidden=256, heads=4, d_ff=704, vocab=64, eps=1e-6, alibi=alibi, max_batch=6,
+                          max_prompt=12, max_full_seq=24)
+    sd, raw = D.random_state_dict(cfg, seed=27)
+    sd["lm_head.weight"] = sd["lm_head.weight"] * 8          # separates the candidates' scores
+    ids = torch.randint(0, cfg.vocab, (2, 6), generator=torch.Generator().manual_seed(12))
+    model = D.Int8Decoder(cfg, sd, device="cuda:0")
+    ref = oracle_decoder(cfg, sd, raw)
+    toks, scores = model.beam_search(ids.to(gpu), 3, 9, eos_token_id=eos, pad_token_id=0)
+    want_t, want_s = ref.beam_search(ids.numpy(), 3, 9, eos=eos, pad_token=0)
+    assert np.array_equal(toks.numpy(), want_t), (toks, want_t)
+    assert np.abs(scores.numpy() - want_s).max() < 2e-2
+    assert model.reorder_state.numel() == 0                   # the driver leaves no reorder behind
+    one, _ = model.beam_search(ids.to(gpu), 1, 5)
+    assert torch.equal(one, D.Int8Decoder(cfg, sd, device="cuda:0").greedy(ids.to(gpu), 5).cpu())
+    with pytest.raises(RuntimeError, match="exceeds max_batch"):
+        model.beam_search(ids.to(gpu), 4, 3)
+
+
 @pytest.mark.parametrize("alibi", [False, True])
 def test_left_padded_batch(gpu, alibi):
     """attention_mask with left padding -> pre_padding_len (modeling_llama.py:276-279): prefill and

@@ -296,3 +296,66 @@ def test_bias_branch_one_token_closed_form():
     plain = O.OracleFFN(g_q, g_s, u_q, u_s, d_q, d_s, g, EPS)
     assert max_rel(plain.forward(x2, False, True), rms(x64 + ffn_core(rms))) < 1e-2      # RMSnorm tail without a bias
     assert max_rel(plain.forward(x2, True, False), ffn_core(rms)) < 1e-2
+
+
+def test_beam_search_against_exhaustive_search():
+    """The checker's beam search over a first-order table model (logits depend on the last token only), where
+    the answer can be enumerated: with num_beams >= V^(T-1) every prefix survives, so the result is the
+    sequence of highest total log-probability among all V^T; with one beam it is the greedy sequence; with an
+    end-of-sequence token the returned score is the length-normalised log-probability of what is returned."""
+    import itertools
+    rng = np.random.default_rng(33)
+    V, T = 5, 3
+    table = rng.standard_normal((V, V)) * 2.0
+    logp = table - np.log(np.exp(table).sum(-1, keepdims=True))
+
+    def step_fn(ids, first, reorder):
+        return table[ids[:, -1]]
+    prompt = np.array([[1, 3], [0, 2]])
+    toks, score = O.beam_search(step_fn, prompt, V ** (T - 1), T)
+    for b in range(2):
+        best = max(itertools.product(range(V), repeat=T),
+                   key=lambda s: logp[prompt[b, -1], s[0]] + logp[s[0], s[1]] + logp[s[1], s[2]])
+        assert tuple(toks[b]) == best
+        total = logp[prompt[b, -1], best[0]] + logp[best[0], best[1]] + logp[best[1], best[2]]
+        assert abs(score[b] - total / (2 + T)) < 1e-9            # length penalty 1: divided by prompt + generated
+    toks1, _ = O.beam_search(step_fn, prompt, 1, 4)
+    for b in range(2):
+        last, greedy = prompt[b, -1], []
+        for _ in range(4):
+            last = int(np.argmax(table[last]))
+            greedy.append(last)
+        assert list(toks1[b]) == greedy
+    # a narrow beam can miss the optimum but never beats it
+    toks2, score2 = O.beam_search(step_fn, prompt, 2, T)
+    assert (score2 <= score + 1e-12).all()
+    # with an end token: what comes back is a closed hypothesis (scored at its length without the end token) or an
+    # open beam, and its score is the one recomputed from the table
+    eos = 4
+    toks3, score3 = O.beam_search(step_fn, prompt, 3, 6, eos=eos, pad_token=-1)
+    for b in range(2):
+        seq = [t for t in toks3[b] if t != -1]
+        assert eos not in seq
+        last, total = prompt[b, -1], 0.0
+        for t in seq:
+            total += logp[last, t]
+            last = t
+        closed = total + logp[last, eos]
+        cands = [closed / (2 + len(seq))] + ([total / (2 + len(seq))] if len(seq) == 6 else [])
+        assert min(abs(score3[b] - c) for c in cands) < 1e-9
+
+
+def test_beam_search_cache_reorder_matches_cacheless_model():
+    """The oracle decoder under beam search (KV caches gathered by the source-beam index at every step) against
+    the same search over the independent model that recomputes every beam's whole sequence without a cache."""
+    hf, orc, rng = make_model(19, batch=6, cap=24)
+    ids = rng.integers(0, 96, (2, 4))
+    hist = {}
+
+    def cacheless(x, first, reorder):
+        hist["ids"] = x if first else np.concatenate([hist["ids"][reorder], x], axis=1)
+        return hf.logits(hist["ids"])[:, -1]
+    want_t, want_s = O.beam_search(cacheless, ids, 3, 6)
+    got_t, got_s = orc.beam_search(ids, 3, 6)
+    assert np.array_equal(got_t, want_t)
+    assert np.abs(got_s - want_s).max() < 2e-2

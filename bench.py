@@ -99,6 +99,13 @@ def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup, probe=Fals
     predecessor's completion counter."""
     st = torch.cuda.current_stream()
     calls = []
+    # the workspace the decoder ops hand to the launches without a prologue (the small-M kernel's k split):
+    # one zero-initialised buffer shared by all launches of the stream, as in eet_amd/ops.py
+    ws_need = max([lib.eet_gemm_w8a16_workspace(M, w.shape[1], w.shape[0], epi)
+                   for layer in weights for name, (w, s, epi) in layer.items() if name not in RMS_LAUNCHES] + [0])
+    if "k_split_ws" not in outs or outs["k_split_ws"].numel() * 4 < ws_need:
+        outs["k_split_ws"] = torch.zeros(max(ws_need // 4, 1), dtype=torch.float32, device=outs["gamma"].device)
+    wsp, wsb = (outs["k_split_ws"].data_ptr(), outs["k_split_ws"].numel() * 4) if ws_need else (None, 0)
     for layer in weights:
         for name, (w, s, epi) in layer.items():
             K, N = w.shape
@@ -132,7 +139,7 @@ def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup, probe=Fals
     else:
         def one_pass():
             for (a, w, s, c, m, n, k, epi, res, gam) in calls:
-                rc = f(a, w, s, c, m, n, k, epi, res, gam, 1e-6, None, 0, sp)
+                rc = f(a, w, s, c, m, n, k, epi, res, gam, 1e-6, None if gam else wsp, 0 if gam else wsb, sp)
                 if rc:
                     raise RuntimeError(lib.eet_last_error().decode())
     for _ in range(warmup):

@@ -27,7 +27,7 @@ SIGNATURES = {
     "eet_gemm_w8a16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _vp]),
     "eet_gemm_w8a16_workspace": (_sz, [_i, _i, _i, _i]),
     "eet_gemm_w8a16_fused": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _f, _vp, _sz, _vp]),
-    "eet_gemm_w8a16_small_m_shape": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "eet_gemm_w8a16_small_m_shape": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "eet_gemm_w8a16_chained": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _f, _i, _vp]),
     "eet_chain_status": (_i, [_vp, _i, _vp]),
     "eet_mmha_decode_workspace": (_sz, [_i, _i, _i, _i]),
@@ -39,10 +39,10 @@ SIGNATURES = {
     "eet_mmha_decode_replayable": (_i, [_vp, _vp, _vp, _l, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp, _i, _i, _vp, _vp,
                                         _sz, _vp]),
     "eet_mmha_int8_decode_replayable": (_i, [_vp, _vp, _f] + [_vp] * 7 + [_i] + [_vp] * 5 + [_i] * 4 + [_vp, _i, _i, _vp,
-                                                                                                 _sz, _vp]),
+                                                                                                 _sz, _vp, _sz, _vp]),
     "eet_mmha_int8_decode_workspace": (_sz, [_i, _i, _i, _i]),
-    "eet_mmha_int8_decode": (_i, [_vp, _vp, _f] + [_vp] * 12 + [_i] * 6 + [_vp, _sz, _vp]),
-    "eet_gated_ffn_int8_decode": (_i, [_vp, _vp, _f] + [_vp] * 6 + [_i] * 4 + [_vp]),
+    "eet_mmha_int8_decode": (_i, [_vp, _vp, _f] + [_vp] * 12 + [_i] * 6 + [_vp, _sz, _vp, _sz, _vp]),
+    "eet_gated_ffn_int8_decode": (_i, [_vp, _vp, _f] + [_vp] * 6 + [_i] * 4 + [_vp, _sz, _vp]),
     "eet_rope_table": (_i, [_vp, _i, _i, _vp]),
     "eet_rmsnorm": (_i, [_vp, _vp, _vp, _i, _i, _f, _vp]),
     "eet_layernorm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _vp]),

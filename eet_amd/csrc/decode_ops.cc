@@ -32,7 +32,8 @@ extern "C" int eet_mmha_int8_decode(const void *x, const void *rms_gamma, float 
                                     const void *qkv_scale, const void *o_w, const void *o_scale, void *k_cache,
                                     void *v_cache, const void *alibi, const int64_t *pad, const float *rope_cos_sin,
                                     void *qkv_buf, void *ctx_buf, void *out, int B, int H, int dh, int hidden,
-                                    int step, int T_cap, void *workspace, size_t workspace_bytes, void *stream)
+                                    int step, int T_cap, void *workspace, size_t workspace_bytes, void *gemm_workspace,
+                                    size_t gemm_workspace_bytes, void *stream)
 {
     EET_REQUIRE(x && rms_gamma && qkv_buf && ctx_buf && out, EET_ERR_INVALID_ARGUMENT,
                 "eet_mmha_int8_decode: null pointer");
@@ -63,12 +64,13 @@ extern "C" int eet_mmha_int8_decode(const void *x, const void *rms_gamma, float 
         return rc;
     // output projection + residual (:260-262, 428-462)
     return eet_gemm_w8a16_fused(ctx_buf, o_w, o_scale, out, B, hidden, inner, EET_EPILOGUE_RESIDUAL, x, nullptr, 0.f,
-                                nullptr, 0, stream);
+                                gemm_workspace, gemm_workspace_bytes, stream);
 }
 
 extern "C" int eet_gated_ffn_int8_decode(const void *x, const void *rms_gamma, float rms_eps, const void *w01,
                                          const void *scale01, const void *w2, const void *scale2, void *act_buf,
-                                         void *out, int B, int hidden, int d_ff, int add_residual, void *stream)
+                                         void *out, int B, int hidden, int d_ff, int add_residual,
+                                         void *gemm_workspace, size_t gemm_workspace_bytes, void *stream)
 {
     EET_REQUIRE(x && rms_gamma && act_buf && out, EET_ERR_INVALID_ARGUMENT, "eet_gated_ffn_int8_decode: null pointer");
     EET_REQUIRE(B > 0 && B <= 32 && hidden > 0 && d_ff > 0, EET_ERR_UNSUPPORTED_SHAPE,
@@ -87,7 +89,7 @@ extern "C" int eet_gated_ffn_int8_decode(const void *x, const void *rms_gamma, f
     // down projection + residual (:122-128, 303-357)
     return eet_gemm_w8a16_fused(act_buf, w2, scale2, out, B, hidden, d_ff,
                                 add_residual ? EET_EPILOGUE_RESIDUAL : EET_EPILOGUE_NONE, add_residual ? x : nullptr,
-                                nullptr, 0.f, nullptr, 0, stream);
+                                nullptr, 0.f, gemm_workspace, gemm_workspace_bytes, stream);
 }
 
 // The same incremental call in its replayable form (see eet_mmha_decode_replayable): recorded once
@@ -98,7 +100,8 @@ extern "C" int eet_mmha_int8_decode_replayable(const void *x, const void *rms_ga
                                                const int64_t *pad, const float *rope_table, void *qkv_buf,
                                                void *ctx_buf, void *out, int B, int H, int dh, int hidden,
                                                const int *step_dev, int step_max, int T_cap, void *workspace,
-                                               size_t workspace_bytes, void *stream)
+                                               size_t workspace_bytes, void *gemm_workspace,
+                                               size_t gemm_workspace_bytes, void *stream)
 {
     EET_REQUIRE(x && rms_gamma && qkv_buf && ctx_buf && out, EET_ERR_INVALID_ARGUMENT,
                 "eet_mmha_int8_decode_replayable: null pointer");
@@ -121,5 +124,5 @@ extern "C" int eet_mmha_int8_decode_replayable(const void *x, const void *rms_ga
                                             workspace, workspace_bytes, stream))
         return rc;
     return eet_gemm_w8a16_fused(ctx_buf, o_w, o_scale, out, B, hidden, inner, EET_EPILOGUE_RESIDUAL, x, nullptr, 0.f,
-                                nullptr, 0, stream);
+                                gemm_workspace, gemm_workspace_bytes, stream);
 }

@@ -196,12 +196,32 @@ __device__ __forceinline__ void mma_batch(const Batch<NT, RG, U> &b, floatx4 (&a
 // weight batches are requested, then the workgroup waits for the producer of A and of the
 // residual rows, reads both with agent-scope loads, writes C with agent-scope stores and
 // signals its own completion; `link` is ignored otherwise.
-template <int NT, int RG, int WAVES, int U, bool RMS, bool CHAIN>
+//
+// MODE kPair2 / kPair4: the k range of a group of NT n-tiles is shared by KS = 2 or 4 workgroups
+// (grid.y = KS), so that a launch whose N leaves one n-tile per CU can give a workgroup NT = KS (or
+// more) n-tiles and still fill the chip: every workgroup reads all M x K / KS activations of its k
+// share, i.e. the L2 -> CU activation traffic of the launch falls by the factor NT.  Each workgroup
+// writes its fp32 tile sums to its slot of `pair.sums` (agent-scope stores), then takes a ticket from
+// the group's counter; the one that arrives LAST adds the others' sums to its own and finishes the
+// tiles (scale, epilogue, store) and puts the counter back to zero.  Nobody waits for anybody.  Slots and
+// counters live in the CALLER's workspace (so calls on different streams never share them): the
+// counters must be zero before the first launch that uses a workspace; every launch leaves them zero.
+struct PairArgs {
+    floatx4 *sums;      // [groups][KS][NT * MT][64]
+    unsigned *tickets;  // [groups], 64 bytes apart
+};
+constexpr int kPlain = 0, kChained = 1, kPair2 = 2, kPair4 = 4;
+constexpr int kPairTiles = 10;   // NT * MT <= 10 tiles per group
+
+template <int NT, int RG, int WAVES, int U, bool RMS, int MODE>
 __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
     _Float16 *__restrict__ C, int M, int N, int K, const _Float16 *__restrict__ residual, int epi,
-    const _Float16 *__restrict__ rms_gamma, float rms_eps, eet::ChainLink link)
+    const _Float16 *__restrict__ rms_gamma, float rms_eps, eet::ChainLink link, PairArgs pair)
 {
+    constexpr bool CHAIN = MODE == kChained, PAIR = MODE == kPair2 || MODE == kPair4;
+    constexpr int KS = PAIR ? MODE : 1;
+    static_assert(!PAIR || (!RMS && NT * ((RG + 1) / 2) <= kPairTiles), "k split: no RMSnorm prologue, at most 10 tiles");
 #if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
     constexpr int MT = (RG + 1) / 2;
     const int lane = threadIdx.x & 63;
@@ -285,10 +305,14 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     // next is issued on every pass, past the end too (where it costs nothing):
     // with a branch around it the compiler has to wait for that request as well
     // before the second multiply, i.e. it empties the pipeline once per pass.
-    const int mine = (ktiles - wave + WAVES - 1) / WAVES;
+    // this workgroup's k-tiles: all of them, or with the k split the share blockIdx.y names
+    const int kt_begin = PAIR ? (int)((long)blockIdx.y * ktiles / KS) : 0;
+    const int kt_end = PAIR ? (int)((long)(blockIdx.y + 1) * ktiles / KS) : ktiles;
+    const int span = kt_end - kt_begin;
+    const int mine = span > wave ? (span - wave + WAVES - 1) / WAVES : 0;
     const int nbatch = mine / U;
     constexpr int STEP = U * WAVES;
-    int kt = wave;
+    int kt = kt_begin + wave;
     if constexpr (CHAIN) {
         // Chained form.  The weights of the first two batches depend on nothing and are requested
         // at once; then the wait for the producer; then the residual rows and the activations of
@@ -336,7 +360,7 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
             mma_batch<NT, RG, U, RMS>(b0, acc, slab, lane, ss);
             kt += STEP;
         }
-        for (; kt < ktiles; kt += WAVES) {
+        for (; kt < kt_end; kt += WAVES) {
             Batch<NT, RG, 1> b;
             load_batch_w<NT, RG, WAVES, 1>(b, wrsrc, wtile, lane, kt, true);
             load_batch_a_chained<NT, RG, WAVES, 1, RMS>(b, arsrc, aoff, gbase, kt, true);
@@ -359,7 +383,7 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
                 kt += STEP;
             }
         }
-        for (; kt < ktiles; kt += WAVES) {
+        for (; kt < kt_end; kt += WAVES) {
             Batch<NT, RG, 1> b;
             load_batch<NT, RG, WAVES, 1, RMS>(b, wrsrc, wtile, lane, abase, gbase, kt, true);
             mma_batch<NT, RG, 1, RMS>(b, acc, slab, lane, ss);
@@ -408,6 +432,42 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         else
             *reinterpret_cast<half4 *>(C + elem) = o;
     };
+    // k split: publish this share's tile sums, take a ticket; all but the last arrival are done, the
+    // last adds the others' sums and goes on to the epilogue.
+    floatx4 whole[kMaxUnits];
+    if constexpr (PAIR) {
+        constexpr int kTiles = NT * MT;
+        const __amdgpu_buffer_rsrc_t prs = __builtin_amdgcn_make_buffer_rsrc(
+            pair.sums + ((size_t)blockIdx.x * KS * kTiles) * 64, 0, (unsigned)KS * kTiles * 64u * 16u, 0x00020000);
+        int i2 = 0;
+        for (int unit = wave; unit < units; unit += WAVES, ++i2) {
+            whole[i2] = tile_sum(unit);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, whole[i2]), prs,
+                                                   (unsigned)(((blockIdx.y * kTiles + unit) * 64 + lane) * 16), 0,
+                                                   kAgentScope);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __shared__ unsigned ticket;
+        __syncthreads();
+        if (threadIdx.x == 0)
+            ticket = __hip_atomic_fetch_add(pair.tickets + blockIdx.x * 16, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (ticket != KS - 1)
+            return;   // the last arrival will find these sums and finish
+        if (threadIdx.x == 0)   // ready for the next launch on this workspace
+            __hip_atomic_store(pair.tickets + blockIdx.x * 16, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        i2 = 0;
+        for (int unit = wave; unit < units; unit += WAVES, ++i2) {
+#pragma unroll
+            for (int o = 1; o < KS; ++o) {
+                const unsigned share = (blockIdx.y + o) % KS;
+                const u32x4 v = __builtin_bit_cast(
+                    u32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                               prs, (unsigned)(((share * kTiles + unit) * 64 + lane) * 16), 0, kAgentScope));
+                whole[i2] += __builtin_bit_cast(floatx4, v);
+            }
+        }
+    }
     int idx = 0;
     for (int unit = wave; unit < units; unit += WAVES, ++idx) {
         const int mt = unit % MT;
@@ -438,7 +498,7 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
             }
         } else {
             const int t = unit / MT;
-            const floatx4 s = tile_sum(unit);
+            const floatx4 s = PAIR ? whole[idx] : tile_sum(unit);
             if (nt0 + t < ntiles && m < M) {
                 const int n = (nt0 + t) * 16 + 4 * g;
                 half4 o;
@@ -458,6 +518,7 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
 
 struct SmallMConfig {
     int nt, waves, u;
+    int ksplit = 1;   // 2: the pair split (nt is 2 then)
 };
 
 template <int NT, int RG, int WAVES, int U, bool RMS>
@@ -465,8 +526,40 @@ int launch_small_m(const GemmArgs &a)
 {
     const int ntiles = a.N / 16;
     dim3 grid((ntiles + NT - 1) / NT), block(WAVES * 64);
-    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U, RMS, false>), grid, block, 0, a.st, a.A, a.Wp, a.scale,
-                       a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, eet::ChainLink{});
+    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U, RMS, kPlain>), grid, block, 0, a.st, a.A, a.Wp, a.scale,
+                       a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, eet::ChainLink{}, PairArgs{});
+    EET_HIP_CHECK(hipGetLastError());
+    return EET_OK;
+}
+
+// Workspace of a k-split launch: the arrival counters, one per group and 64 bytes apart, in a region of
+// fixed size (so that calls of different shapes on one workspace keep their counters in the same, always
+// zero, place), then the exchange slots.
+constexpr int kSplitMaxGroups = 512;
+constexpr size_t kSplitTicketBytes = (size_t)kSplitMaxGroups * 64;
+size_t k_split_workspace(int M, int N, int nt, int ks)
+{
+    const int groups = (N / 16 + nt - 1) / nt, mt = M <= 16 ? 1 : 2;
+    return kSplitTicketBytes + (size_t)groups * ks * nt * mt * 1024;
+}
+
+// The k split (kernel comment above): NT n-tiles per group of KS workgroups, each a share of the k range.
+template <int NT, int RG, int WAVES, int U, int KS>
+int launch_small_m_pair(const GemmArgs &a)
+{
+    const int groups = (a.N / 16 + NT - 1) / NT;
+    EET_REQUIRE(groups <= kSplitMaxGroups, EET_ERR_UNSUPPORTED_SHAPE, "eet_gemm_w8a16: the k split takes at most %d groups",
+                kSplitMaxGroups);
+    EET_REQUIRE(a.ws != nullptr && reinterpret_cast<uintptr_t>(a.ws) % 16 == 0 &&
+                    a.ws_bytes >= k_split_workspace(a.M, a.N, NT, KS),
+                EET_ERR_WORKSPACE, "eet_gemm_w8a16: the k split needs a 16-byte aligned workspace of %zu bytes, %zu given",
+                k_split_workspace(a.M, a.N, NT, KS), a.ws_bytes);
+    PairArgs pa;
+    pa.tickets = static_cast<unsigned *>(a.ws);
+    pa.sums = reinterpret_cast<floatx4 *>(static_cast<char *>(a.ws) + kSplitTicketBytes);
+    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U, false, KS>), dim3(groups, KS), dim3(WAVES * 64), 0, a.st,
+                       a.A, a.Wp, a.scale, a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps,
+                       eet::ChainLink{}, pa);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
@@ -482,13 +575,13 @@ int launch_small_m_chained(const GemmArgs &a)
     bool any_order = false;
     if (int rc = eet::chain_link("eet_gemm_w8a16_chained", a.chain, grid.x, a.st, &link, &any_order))
         return rc;
-    auto kern = w8a16_small_m_kernel<NT, RG, WAVES, U, RMS, true>;
+    auto kern = w8a16_small_m_kernel<NT, RG, WAVES, U, RMS, kChained>;
     if (any_order)
         hipExtLaunchKernelGGL(kern, grid, block, 0, a.st, nullptr, nullptr, hipExtAnyOrderLaunch, a.A, a.Wp, a.scale,
-                              a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, link);
+                              a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, link, PairArgs{});
     else
         hipLaunchKernelGGL(kern, grid, block, 0, a.st, a.A, a.Wp, a.scale, a.C, a.M, a.N, a.K, a.residual, a.epi,
-                           a.rms_gamma, a.rms_eps, link);
+                           a.rms_gamma, a.rms_eps, link, PairArgs{});
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
@@ -523,6 +616,22 @@ int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a, bool dry)
     if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_) {                            \
         if constexpr (small_m_fits(NT_, RG, W_, U_))                                  \
             return dry ? EET_OK : launch_small_m<NT_, RG, W_, U_, true>(a);           \
+    }
+    if (cfg.ksplit > 1) {
+        // the k split: no RMSnorm prologue, no SwiGLU epilogue, not chained
+        if (a.rms_gamma != nullptr || a.epi == kEpiSwiglu || a.chain != eet::kChainOff)
+            return kNoVariant;
+#define EET_CASE_SPLIT(NT_, W_, U_, KS_)                                                     \
+    if (cfg.nt == NT_ && cfg.waves == W_ && cfg.u == U_ && cfg.ksplit == KS_) {              \
+        if constexpr (small_m_fits(NT_, RG, W_, U_) && NT_ * ((RG + 1) / 2) <= kPairTiles)   \
+            return dry ? EET_OK : launch_small_m_pair<NT_, RG, W_, U_, KS_>(a);              \
+    }
+        EET_CASE_SPLIT(2, 8, 1, 2) EET_CASE_SPLIT(2, 8, 2, 2) EET_CASE_SPLIT(2, 4, 2, 2)
+        EET_CASE_SPLIT(4, 8, 1, 4) EET_CASE_SPLIT(4, 4, 2, 4) EET_CASE_SPLIT(4, 4, 1, 4) EET_CASE_SPLIT(4, 8, 1, 2)
+        EET_CASE_SPLIT(5, 8, 1, 4) EET_CASE_SPLIT(5, 4, 2, 4) EET_CASE_SPLIT(5, 4, 1, 4)
+        EET_CASE_SPLIT(3, 8, 1, 2) EET_CASE_SPLIT(3, 8, 1, 4) EET_CASE_SPLIT(6, 8, 1, 2)
+#undef EET_CASE_SPLIT
+        return kNoVariant;
     }
     if (a.chain != eet::kChainOff) {
         // chained kernels exist for the launch shapes pick_small_m can return
@@ -572,10 +681,37 @@ int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a, bool dry)
 // (M = 32: 20.1 against 28.1 us).  The SwiGLU epilogue needs an even NT (gate / up
 // pairs).  One n-tile per workgroup runs with 16 wavefronts when there are few
 // workgroups (more loads in flight per CU).
-SmallMConfig pick_small_m(int M, int N, int K, int epi, bool rms)
+// The k split for the launches without a prologue (O and down projections), where N leaves about one
+// n-tile per CU and NT cannot grow without idling CUs.  Measured on MI355X against the table's choice
+// (us; residual epilogue; 24 matrices in rotation):
+//   N = 4096 (256 n-tiles)            K = 4096: M=16 6.83 -> 6.35 (NT 2, 2 shares)   M=32 8.38 -> 7.38 (NT 2, 2 shares)
+//                                     K = 11008: M=16 11.93 -> 10.91 (NT 4, 4 shares) M=32 17.03 -> 13.01 (NT 4, 4 shares)
+//                                     M <= 8: no split (5.85 / 9.87 against 6.22 / 10.29)
+//   N = 5120 (320 n-tiles, 1.25 per CU: NT 5 with 4 shares makes 256 equal workgroups)
+//                                     K = 5120: M=8 7.83 -> 7.67, M=16 9.18 -> 7.94, M=32 11.75 -> 12.29 (not taken)
+//                                     K = 13696: M=8 16.43 -> 14.34, M=16 19.53 -> 14.41, M=32 25.27 -> 19.74
+// Other channel counts keep the table's choice.
+bool pick_k_split(int M, int ntiles, int K, SmallMConfig *out)
+{
+    if (ntiles == 256 && M > 8) {
+        if (K <= 8192)
+            *out = M <= 16 ? SmallMConfig{2, 4, 2, 2} : SmallMConfig{2, 8, 1, 2};
+        else
+            *out = M <= 16 ? SmallMConfig{4, 4, 1, 4} : SmallMConfig{4, 8, 1, 4};
+        return true;
+    }
+    if (ntiles == 320 && !(M > 16 && K <= 8192)) {
+        *out = SmallMConfig{5, 8, 1, 4};
+        return true;
+    }
+    return false;
+}
+
+SmallMConfig pick_small_m(int M, int N, int K, int epi, bool rms, bool may_split)
 {
     const int ntiles = N / 16;
-    (void)K;
+    if (SmallMConfig split; may_split && !rms && epi != kEpiSwiglu && pick_k_split(M, ntiles, K, &split))
+        return split;
     int best_nt = 0;
     double best = 0.0;
     for (int nt : {1, 2, 3, 4, 6, 8}) {
@@ -617,11 +753,16 @@ SmallMConfig resolve_small_m(const GemmArgs &a)
 {
     const eet::Tuning &tune = eet::tuning();
     if (tune.has_small_m && (a.epi != kEpiSwiglu || tune.small_m_nt % 2 == 0)) {
-        const SmallMConfig forced{tune.small_m_nt, tune.small_m_waves, tune.small_m_u};
+        const SmallMConfig forced{tune.small_m_nt, tune.small_m_waves, tune.small_m_u, tune.small_m_ksplit};
         if (dispatch_by_rows(forced, a, true) == EET_OK)
             return forced;
     }
-    return pick_small_m(a.M, a.N, a.K, a.epi, a.rms_gamma != nullptr);
+    // the k split runs out of the caller's workspace: without a sufficient one the table's choice stands
+    SmallMConfig cfg = pick_small_m(a.M, a.N, a.K, a.epi, a.rms_gamma != nullptr, a.chain == eet::kChainOff);
+    if (cfg.ksplit > 1 && (a.ws == nullptr || reinterpret_cast<uintptr_t>(a.ws) % 16 != 0 ||
+                           a.ws_bytes < k_split_workspace(a.M, a.N, cfg.nt, cfg.ksplit)))
+        cfg = pick_small_m(a.M, a.N, a.K, a.epi, a.rms_gamma != nullptr, false);
+    return cfg;
 }
 
 int run_small_m(const GemmArgs &a)
@@ -633,8 +774,9 @@ int run_small_m(const GemmArgs &a)
     const SmallMConfig cfg = resolve_small_m(a);
     const int rc = dispatch_by_rows(cfg, a, false);   // a launch failure is returned as it is
     if (rc == kNoVariant)
-        return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16: no small-M kernel for nt=%d waves=%d u=%d (M=%d%s)",
-                         cfg.nt, cfg.waves, cfg.u, a.M, a.rms_gamma ? ", RMSnorm prologue" : "");
+        return eet::fail(EET_ERR_INVALID_ARGUMENT,
+                         "eet_gemm_w8a16: no small-M kernel for nt=%d waves=%d u=%d ksplit=%d (M=%d%s)", cfg.nt, cfg.waves,
+                         cfg.u, cfg.ksplit, a.M, a.rms_gamma ? ", RMSnorm prologue" : "");
     return rc;
 }
 
@@ -702,9 +844,10 @@ extern "C" int eet_gemm_w8a16(const void *A, const void *Wpacked, const void *sc
 }
 
 extern "C" int eet_gemm_w8a16_small_m_shape(int M, int N, int K, int epilogue, int rms_prologue, int *nt, int *waves,
-                                            int *k_tiles_per_batch)
+                                            int *k_tiles_per_batch, int *k_split)
 {
-    EET_REQUIRE(nt && waves && k_tiles_per_batch, EET_ERR_INVALID_ARGUMENT, "eet_gemm_w8a16_small_m_shape: null pointer");
+    EET_REQUIRE(nt && waves && k_tiles_per_batch && k_split, EET_ERR_INVALID_ARGUMENT,
+                "eet_gemm_w8a16_small_m_shape: null pointer");
     EET_REQUIRE(M >= 1 && M <= 32 && N > 0 && K > 0 && K % 64 == 0 && N % 16 == 0, EET_ERR_UNSUPPORTED_SHAPE,
                 "eet_gemm_w8a16_small_m_shape: not a shape the small-M kernel takes (M=%d N=%d K=%d)", M, N, K);
     GemmArgs a{};
@@ -712,14 +855,21 @@ extern "C" int eet_gemm_w8a16_small_m_shape(int M, int N, int K, int epilogue, i
     static const _Float16 kSomeGamma = 0;
     a.rms_gamma = rms_prologue ? &kSomeGamma : nullptr;   // only tested against null
     const SmallMConfig cfg = resolve_small_m(a);
-    *nt = cfg.nt, *waves = cfg.waves, *k_tiles_per_batch = cfg.u;
+    *nt = cfg.nt, *waves = cfg.waves, *k_tiles_per_batch = cfg.u, *k_split = cfg.ksplit;
     return EET_OK;
 }
 
 extern "C" size_t eet_gemm_w8a16_workspace(int M, int N, int K, int epilogue)
 {
-    if (M <= 32 || N <= 0 || K <= 0 || K % 64 != 0 || N % 16 != 0)
+    if (M <= 0 || N <= 0 || K <= 0 || K % 64 != 0 || N % 16 != 0)
         return 0;
+    if (M <= 32) {   // the small-M kernel's k split (launches without the RMSnorm prologue)
+        const eet::Tuning &tune = eet::tuning();
+        SmallMConfig cfg = pick_small_m(M, N, K, epilogue, false, true);
+        if (tune.has_small_m && tune.small_m_ksplit > 1)
+            cfg = SmallMConfig{tune.small_m_nt, tune.small_m_waves, tune.small_m_u, tune.small_m_ksplit};
+        return cfg.ksplit > 1 ? k_split_workspace(M, N, cfg.nt, cfg.ksplit) : 0;
+    }
     return eet::large_m_workspace(M, N, K, epilogue);
 }
 

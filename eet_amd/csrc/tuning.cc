@@ -19,8 +19,10 @@ int apply(const char *name, const char *value)
         t.has_small_m = false;
         if (clear)
             return EET_OK;
-        if (std::sscanf(value, "%d,%d,%d", &t.small_m_nt, &t.small_m_waves, &t.small_m_u) != 3)
-            return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_set_tuning: %s wants \"nt,waves,u\", got \"%s\"", name, value);
+        t.small_m_ksplit = 1;
+        if (std::sscanf(value, "%d,%d,%d,%d", &t.small_m_nt, &t.small_m_waves, &t.small_m_u, &t.small_m_ksplit) < 3)
+            return eet::fail(EET_ERR_INVALID_ARGUMENT, "eet_set_tuning: %s wants \"nt,waves,u[,ksplit]\", got \"%s\"", name,
+                             value);
         t.has_small_m = true;
         return EET_OK;
     }

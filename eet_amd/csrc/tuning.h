@@ -9,9 +9,9 @@
 namespace eet {
 
 struct Tuning {
-    // EET_GEMM_SMALL_M_CONFIG = "nt,waves,u"
+    // EET_GEMM_SMALL_M_CONFIG = "nt,waves,u[,ksplit]" (ksplit 2: the pair split, with nt = 2)
     bool has_small_m = false;
-    int small_m_nt = 0, small_m_waves = 0, small_m_u = 0;
+    int small_m_nt = 0, small_m_waves = 0, small_m_u = 0, small_m_ksplit = 1;
     // EET_GEMM_LARGE_M_TILE = "tm,tn[,ksplit]"
     bool has_large_m = false;
     int large_m_tm = 0, large_m_tn = 0, large_m_ksplit = 0;  // ksplit 0: not given

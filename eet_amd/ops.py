@@ -60,11 +60,12 @@ class _Workspaces:
         self._bufs = {}
         self._recorders = []
 
-    def get(self, name, numel, dtype, device):
+    def get(self, name, numel, dtype, device, zero=False):
         key = (name, str(device), dtype)
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < numel:
-            buf = torch.empty(max(int(numel), 1), dtype=dtype, device=device)
+            alloc = torch.zeros if zero else torch.empty      # zero: a buffer whose first use needs zeros
+            buf = alloc(max(int(numel), 1), dtype=dtype, device=device)
             self._bufs[key] = buf
         for handed in self._recorders:
             handed.append(buf)
@@ -227,6 +228,16 @@ def linear_bytes(M, K, N, epilogue=EPI_NONE):
 RMS_FUSE_MAX_M = 32     # the RMSnorm prologue exists in the small-M kernel only
 
 
+def _k_split_ws(M, N, K, epilogue, device):
+    """(pointer, bytes) of the small-M kernel's k-split workspace for this call, or (None, 0).  A buffer of its
+    own, zero when created (the arrival counters at its start must start at zero; every call leaves them so)."""
+    need = lib().eet_gemm_w8a16_workspace(M, N, K, epilogue) if M <= RMS_FUSE_MAX_M else 0
+    if not need:
+        return None, 0
+    buf = workspaces.get("gemm_small_m_k_split", (need + 3) // 4, torch.float32, device, zero=True)
+    return buf.data_ptr(), buf.numel() * 4
+
+
 def _gemm(a, w, scale, out, M, N, K, epilogue=EPI_NONE, residual=None, rms_gamma=None, rms_eps=0.0):
     L = lib()
     ws, ws_bytes = None, 0
@@ -234,6 +245,8 @@ def _gemm(a, w, scale, out, M, N, K, epilogue=EPI_NONE, residual=None, rms_gamma
         ws_bytes = L.eet_gemm_w8a16_workspace(M, N, K, epilogue)
         if ws_bytes:
             ws = workspaces.get("gemm_split_k", ws_bytes // 4, torch.float32, a.device).data_ptr()
+    elif rms_gamma is None:   # launches without a prologue may share a tile group's k range among workgroups
+        ws, ws_bytes = _k_split_ws(M, N, K, epilogue, a.device)
     check(L.eet_gemm_w8a16_fused(a.data_ptr(), w.data_ptr(), scale.data_ptr(), out.data_ptr(), M, N, K,
                                  epilogue, residual.data_ptr() if residual is not None else None,
                                  rms_gamma.data_ptr() if rms_gamma is not None else None, rms_eps, ws, ws_bytes,
@@ -438,7 +451,7 @@ class _MmhaInt8:
                     self.v_cache.data_ptr(), _ptr(alibi), ld, _ptr(pad),
                     self.rope_table.data_ptr() if self._rope else None, qkv.data_ptr(), cbuf.data_ptr(), out.data_ptr(),
                     B, H, dh, hidden, rs.step_dev.data_ptr(), rs.step_max, self.t_cap, ws.data_ptr(), ws.numel() * 4,
-                    _stream()), "eet_mmha_int8_decode_replayable")
+                    *_k_split_ws(B, hidden, self.inner, EPI_RESIDUAL, dev), _stream()), "eet_mmha_int8_decode_replayable")
                 self._keep = (x, pad, alibi, reorder)
                 return out[: M * hidden].view(B, S, hidden)
             rope = self.rope_table.data_ptr() + (self.step - 1) * dh * 4 if self._rope else None
@@ -460,7 +473,8 @@ class _MmhaInt8:
                                          self.o_s.data_ptr(), self.k_cache.data_ptr(), self.v_cache.data_ptr(),
                                          _ptr(alibi), _ptr(pad), rope, qkv.data_ptr(), cbuf.data_ptr(),
                                          out.data_ptr(), B, H, dh, hidden, self.step, self.t_cap, ws.data_ptr(),
-                                         ws.numel() * 4, _stream()), "eet_mmha_int8_decode")
+                                         ws.numel() * 4, *_k_split_ws(B, hidden, self.inner, EPI_RESIDUAL, dev),
+                                         _stream()), "eet_mmha_int8_decode")
             self._keep = (x, pad, alibi, reorder)  # inputs of kernels still in flight
             return out[: M * hidden].view(B, S, hidden)
         if self.with_bias:
@@ -611,7 +625,10 @@ class GatedFeedForwardNetworkInt8:
             check(lib().eet_gated_ffn_int8_decode(x.data_ptr(), self.gamma.data_ptr(), desc.layernorm_eps,
                                                   self.w01.data_ptr(), self.s01.data_ptr(), self.w2.data_ptr(),
                                                   self.s2.data_ptr(), act.data_ptr(), out.data_ptr(), M, hidden,
-                                                  self.d_ff, 1 if add_residual else 0, _stream()),
+                                                  self.d_ff, 1 if add_residual else 0,
+                                                  *_k_split_ws(M, hidden, self.d_ff,
+                                                               EPI_RESIDUAL if add_residual else EPI_NONE, dev),
+                                                  _stream()),
                   "eet_gated_ffn_int8_decode")
             self._keep = x
             return out[: M * hidden].view(B, S, hidden)

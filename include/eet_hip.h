@@ -49,7 +49,7 @@ int eet_packed_layout_version(void);
 
 /* Overrides one of the library's launch-shape tables, for sweeps and for tests
  * that run every kernel variant; value NULL or "" restores the table.  Keys:
- *   EET_GEMM_SMALL_M_CONFIG "nt,waves,u"       EET_GEMM_LARGE_M_TILE "tm,tn[,ksplit]"
+ *   EET_GEMM_SMALL_M_CONFIG "nt,waves,u[,ksplit]"   EET_GEMM_LARGE_M_TILE "tm,tn[,ksplit]"
  *   EET_MMHA_NSPLIT / EET_MMHA_THREADS / EET_MMHA_UNROLL "n"
  *   EET_PREFILL_LEGACY "1" (register-staged prefill attention at head size 128)
  *   EET_PREFILL_SHAPE "1" | "2" (launch shape of the head-size-128 prefill kernel)
@@ -114,10 +114,21 @@ int eet_quantize_pack_device(const void *w, int w_dtype, size_t K, size_t N, int
  * M <= 32 takes the HBM-streaming small-M kernel, larger M the LDS-staged MFMA
  * kernel.  The workspace is optional (NULL / 0 accepted): with
  * eet_gemm_w8a16_workspace(M, N, K, epilogue) bytes of 16-byte aligned device
- * memory the library may split the k range of a launch that has too few tiles to
- * fill the chip (M in the tens to hundreds) and add the parts in a second small
- * kernel -- the reference's split-k workspace, which its callers never pass
- * (fpA_intB_gemm_template.h:443-495, cutlass_heuristic.cc:80-84).
+ * memory the library may split the k range of a launch -- the reference's
+ * split-k workspace, which its callers never pass
+ * (fpA_intB_gemm_template.h:443-495, cutlass_heuristic.cc:80-84):
+ *   M > 32   a launch that has too few tiles to fill the chip (M in the tens to
+ *            hundreds): raw fp32 sums, added in a second small kernel;
+ *   M <= 32  a launch without the RMSnorm prologue whose N leaves about one 16-channel
+ *            tile per CU (the O and down projections at N = 4096 / 5120): 2 or 4
+ *            workgroups share a group of tiles, exchange their fp32 sums through the
+ *            workspace and the last one to arrive finishes them -- one launch.
+ *            For this use the first 32 KiB of the workspace (its arrival counters)
+ *            must be ZERO before the first call that is handed the workspace; every
+ *            call leaves them zero.  Keep such a workspace for
+ *            M <= 32 calls only (an M > 32 call writes partial sums over the
+ *            counters), and never hand one workspace to two calls that can overlap
+ *            in time.
  * Replaces fastertransformer::gemm_fp16_int_bias_act<uint8_t>
  * (3rdparty/cutlass_kernels/fpA_intB_gemm.cu:35-62) as called with
  * bias = nullptr and no activation from csrc/op/llama_mmha.cpp:313-337,
@@ -153,13 +164,14 @@ int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, 
                          size_t workspace_bytes, void *stream);
 
 /* The launch shape the small-M kernel (1 <= M <= 32) runs a call with: n-tiles per
- * workgroup, wavefronts per workgroup, k-tiles per register batch -- the tuning
+ * workgroup, wavefronts per workgroup, k-tiles per register batch, and how many
+ * workgroups share a tile's k range (1, or 2 for the pair split) -- the tuning
  * override EET_GEMM_SMALL_M_CONFIG when a kernel of that shape exists for the
  * call, otherwise the table's choice.  For sweeps and for tests that must know
  * which variant ran.  The reference's counterpart is the CutlassGemmConfig its
  * heuristic returns (cutlass_heuristic.cc:106-207). */
 int eet_gemm_w8a16_small_m_shape(int M, int N, int K, int epilogue, int rms_prologue, int *nt,
-                                 int *waves, int *k_tiles_per_batch);
+                                 int *waves, int *k_tiles_per_batch, int *k_split);
 
 /* Chained launches (1 <= M <= 32): eet_gemm_w8a16_fused for a sequence of launches
  * in which each reads what the previous one wrote -- the decode step of
@@ -306,6 +318,9 @@ int eet_kv_cache_reorder(const void *k_src, const void *v_src, void *k_dst, void
  * [B][3*H*dh] and ctx_buf [B][H*dh] are scratch; out [B][hidden] must not
  * alias x.  Weights are packed int8 [hidden][3*H*dh] and [H*dh][hidden] with
  * their fp16 scales; the other arguments are those of eet_mmha_decode.
+ * gemm_workspace: optional (NULL / 0), the eet_gemm_w8a16 workspace of the output
+ * projection, eet_gemm_w8a16_workspace(B, hidden, H*dh, EET_EPILOGUE_RESIDUAL) bytes
+ * under that function's rules (counters zero before first use).
  * Replaces LlamaMmha::forward_inc (csrc/op/llama_mmha.cpp:202-266) and
  * BaichuanMmha::forward_inc (csrc/op/baichuan_mmha.cpp:166-216) without the
  * beam reorder, which stays a separate call (eet_kv_cache_reorder). */
@@ -315,18 +330,22 @@ int eet_mmha_int8_decode(const void *x, const void *rms_gamma, float rms_eps, co
                          void *k_cache, void *v_cache, const void *alibi, const int64_t *pad,
                          const float *rope_cos_sin, void *qkv_buf, void *ctx_buf, void *out,
                          int B, int H, int dh, int hidden, int step, int T_cap, void *workspace,
-                         size_t workspace_bytes, void *stream);
+                         size_t workspace_bytes, void *gemm_workspace, size_t gemm_workspace_bytes,
+                         void *stream);
 
 /* The gated FFN sub-layer for B <= 32 rows, both launches from one call:
  * RMSnorm + gate and up projections + SwiGLU (w01 / scale01: gate and up
  * interleaved by 16-channel tile, [hidden][2*d_ff]), then the down projection
  * (+ x when add_residual).  act_buf [B][d_ff] is scratch; out [B][hidden] must
- * not alias x.  Replaces GatedFeedForwardNetworkInt8::forward
+ * not alias x.  gemm_workspace: optional (NULL / 0), the eet_gemm_w8a16 workspace of
+ * the down projection, eet_gemm_w8a16_workspace(B, hidden, d_ff, epilogue) bytes under
+ * that function's rules.  Replaces GatedFeedForwardNetworkInt8::forward
  * (csrc/op/gated_ffn_int8.cpp:98-132) at decode sizes. */
 int eet_gated_ffn_int8_decode(const void *x, const void *rms_gamma, float rms_eps, const void *w01,
                               const void *scale01, const void *w2, const void *scale2,
                               void *act_buf, void *out, int B, int hidden, int d_ff,
-                              int add_residual, void *stream);
+                              int add_residual, void *gemm_workspace, size_t gemm_workspace_bytes,
+                              void *stream);
 
 /* Causal prefill attention over the prompt, reading K and V from the caches
  * filled by eet_qkv_split.  q [B][H][S][dh]; ctx [B][S][H*dh]; alibi NULL or
@@ -369,7 +388,7 @@ int eet_mmha_int8_decode_replayable(const void *x, const void *rms_gamma, float 
                                     const float *rope_table, void *qkv_buf, void *ctx_buf, void *out,
                                     int B, int H, int dh, int hidden, const int *step_dev,
                                     int step_max, int T_cap, void *workspace, size_t workspace_bytes,
-                                    void *stream);
+                                    void *gemm_workspace, size_t gemm_workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

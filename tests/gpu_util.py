@@ -46,7 +46,8 @@ def gemm_workspace(M, N, K, epi, device, min_bytes=0):
     need = max(lib().eet_gemm_w8a16_workspace(M, N, K, epi), min_bytes)
     if not need:
         return None, 0, None
-    buf = torch.empty(need // 4, dtype=torch.float32, device=device)
+    # zero-filled: the small-M k split keeps its arrival counters at the start of the workspace
+    buf = torch.zeros((need + 3) // 4, dtype=torch.float32, device=device)
     return buf.data_ptr(), need, buf
 
 

@@ -59,8 +59,13 @@ def test_device_entry_points_validate_before_launch():
     assert L.eet_gemm_w8a16(p, p, p, p, 1, 24, 64, None, 0, None) == -2       # N % 16
     assert b"K % 64" in L.eet_last_error()
     assert L.eet_gemm_w8a16(p, p, p, p, 0, 16, 64, None, 0, None) == 0        # empty batch: nothing to do
-    # split-k workspace: none for the small-M kernel or once the tiles fill the chip, ksplit x M x N fp32 between
-    assert L.eet_gemm_w8a16_workspace(32, 4096, 4096, 0) == 0
+    # split-k workspace: none once the tiles fill the chip, ksplit x M x N fp32 for M in the tens to hundreds;
+    # the small-M kernel's k split: counters + exchange slots for N = 4096 / 5120 at the rows that split
+    assert L.eet_gemm_w8a16_workspace(8, 4096, 4096, 0) == 0 and L.eet_gemm_w8a16_workspace(8, 12288, 4096, 0) == 0
+    assert L.eet_gemm_w8a16_workspace(32, 4096, 4096, 1) == 32768 + 128 * 2 * 2 * 2 * 1024     # counters + NT 2, 2 shares, 2 m-tiles
+    assert L.eet_gemm_w8a16_workspace(16, 4096, 11008, 1) == 32768 + 64 * 4 * 4 * 1 * 1024      # NT 4, 4 shares
+    assert L.eet_gemm_w8a16_workspace(8, 5120, 13696, 1) == 32768 + 64 * 4 * 5 * 1 * 1024       # NT 5, 4 shares
+    assert L.eet_gemm_w8a16_workspace(32, 4096, 4096, 2) == 0                                     # not with SwiGLU
     assert L.eet_gemm_w8a16_workspace(2048, 4096, 4096, 0) == 0
     need = L.eet_gemm_w8a16_workspace(64, 4096, 11008, 0)
     assert need >= 2 * 64 * 4096 * 4 and need % (64 * 4096 * 4) == 0
@@ -75,13 +80,13 @@ def test_device_entry_points_validate_before_launch():
     assert L.eet_mmha_decode(p, None, None, 0, p, p, p, None, None, 1, 8, 128, 1100, 1153, None, None, 0, None) == -4
     # operator-level decode calls: argument checks happen before any launch
     assert L.eet_mmha_int8_decode(None, p, 1e-6, p, p, p, p, p, p, None, None, None, p, p, p, 1, 1, 128, 128, 1, 8,
-                                  None, 0, None) == -1
+                                  None, 0, None, 0, None) == -1
     assert L.eet_mmha_int8_decode(p, p, 1e-6, p, p, p, p, p, p, None, None, None, p, p, p, 33, 1, 128, 128, 1, 8,
-                                  None, 0, None) == -2                       # more than 32 rows
+                                  None, 0, None, 0, None) == -2              # more than 32 rows
     assert L.eet_mmha_int8_decode(p, p, 1e-6, p, p, p, p, p, p, None, None, None, p, p, p, 1, 1, 128, 128, 1, 8,
-                                  None, 0, None) == -1                       # out aliases x
-    assert L.eet_gated_ffn_int8_decode(p, p, 1e-6, p, p, p, p, p, None, 1, 128, 256, 1, None) == -1
-    assert L.eet_gated_ffn_int8_decode(p, p, 1e-6, p, p, p, p, p, p, 40, 128, 256, 1, None) == -2
+                                  None, 0, None, 0, None) == -1              # out aliases x
+    assert L.eet_gated_ffn_int8_decode(p, p, 1e-6, p, p, p, p, p, None, 1, 128, 256, 1, None, 0, None) == -1
+    assert L.eet_gated_ffn_int8_decode(p, p, 1e-6, p, p, p, p, p, p, 40, 128, 256, 1, None, 0, None) == -2
     assert L.eet_mmha_int8_decode_workspace(8, 32, 128, 1100) == L.eet_mmha_decode_workspace(8, 32, 128, 1100)
     assert L.eet_rope_table(None, 4, 128, None) == -1
     assert L.eet_rmsnorm(p, p, p, 1, 20000, 1e-6, None) == -2
@@ -146,7 +151,8 @@ def test_tuning_keys():
     """Every documented tuning key is accepted and cleared (host state only, no GPU); malformed values and
     unknown keys are refused with a message."""
     L = _lib.lib()
-    for name, value in [("EET_GEMM_SMALL_M_CONFIG", "2,8,1"), ("EET_GEMM_LARGE_M_TILE", "4,4"),
+    for name, value in [("EET_GEMM_SMALL_M_CONFIG", "2,8,1"), ("EET_GEMM_SMALL_M_CONFIG", "2,8,1,2"),
+                        ("EET_CHAIN_SPIN_LIMIT", "0"), ("EET_CHAIN_SLEEP", "4"), ("EET_GEMM_LARGE_M_TILE", "4,4"),
                         ("EET_GEMM_LARGE_M_TILE", "2,2,4"), ("EET_MMHA_NSPLIT", "2"), ("EET_MMHA_THREADS", "256"),
                         ("EET_MMHA_UNROLL", "4"), ("EET_PREFILL_LEGACY", "1"), ("EET_PREFILL_SHAPE", "2")]:
         assert L.eet_set_tuning(name.encode(), value.encode()) == 0, L.eet_last_error()

@@ -96,6 +96,15 @@ def test_large_m_path(gpu):
         assert_close(c.cpu().numpy(), O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32), what=f"M={M}")
 
 
+def small_m_shape(M, N, K, epi, rms):
+    """(n-tiles per workgroup, wavefronts, k-tiles per batch, k split) the library runs this call with."""
+    import ctypes
+    from eet_amd._lib import check, lib
+    v = [ctypes.c_int(0) for _ in range(4)]
+    check(lib().eet_gemm_w8a16_small_m_shape(M, N, K, epi, 1 if rms else 0, *[ctypes.byref(x) for x in v]))
+    return tuple(x.value for x in v)
+
+
 SMALL_M_SHAPES = ["1,8,2", "1,16,2", "1,16,1", "2,8,2", "2,8,1", "3,8,1", "4,8,1", "6,8,1", "8,8,1"]   # NT, wavefronts, k-tiles per batch
 
 
@@ -108,7 +117,17 @@ def test_small_m_launch_shapes(gpu, tuning, cfg):
     from eet_amd.ops import interleave_gate_up
     tuning("EET_GEMM_SMALL_M_CONFIG", cfg)
     eps = 1e-6
+    want_shape = tuple(int(v) for v in cfg.split(",")) + (1,)
     for (M, K, N) in [(5, 576, 208), (16, 2752, 1104), (27, 704, 400)]:
+        # the override really selects the kernel that runs (no silent fall-back to the table's choice) ...
+        nt, waves, u = want_shape[:3]
+        rg = (M + 7) // 8 if M <= 16 else 4
+        # ... where a kernel of that shape can exist: the activation slabs of all wavefronts within 64 KiB,
+        # the reduction buffer within 144 KiB (the library's own budget), and an even NT for gate / up pairs
+        exists = waves * u * rg * 1024 <= 65536 and waves * nt * ((rg + 1) // 2) * 1024 <= 147456
+        assert (small_m_shape(M, N, K, 0, False) == want_shape) == exists, (cfg, M)
+        assert (small_m_shape(M, N, K, 1, True) == want_shape) == exists, (cfg, M)
+        assert (small_m_shape(M, 2 * (N // 2 + 8), K, 2, True) == want_shape) == (exists and nt % 2 == 0), (cfg, M)
         x, u, p, s = make(M, K, N, M + K + N)
         g = torch.Generator().manual_seed(M)
         gamma = (1 + 0.1 * torch.randn(K, generator=g)).half()
@@ -142,6 +161,30 @@ PROLOGUE_BOUNDS = {(1, 256, 64, 0): 1e-3,          # [3.5e-6]
                    (16, 1024, 176, 0): 1e-3,       # [3.0e-4]
                    (32, 512, 96, 2): 1e-3,         # [6.4e-5]
                    (5, 11008, 4096, 1): 2.0e-3}    # [1.30e-3]  K = 11008 behind one moved rounding
+
+@pytest.mark.parametrize("cfg", ["2,8,1,2", "2,8,2,2", "4,8,1,4", "5,8,1,4", "4,4,2,4"])
+def test_pair_split(gpu, tuning, cfg):
+    """The k split (2 or 4 workgroups share a group of n-tiles, each takes a share of the k range, the one
+    that arrives last adds the others' fp32 sums and finishes): forced through the tuning override, at the
+    O / down shapes of both decoders and on ragged ones (k-tile and n-tile counts that do not divide), plain
+    and with the residual epilogue, twice in a row (the tickets only ever grow)."""
+    tuning("EET_GEMM_SMALL_M_CONFIG", cfg)
+    for (M, K, N) in [(32, 4096, 4096), (16, 11008, 4096), (8, 5120, 5120), (32, 13696, 5120), (27, 4160, 4112),
+                      (3, 192, 48)]:
+        assert small_m_shape(M, N, K, 1, False) == tuple(int(v) for v in cfg.split(","))
+        x, u, p, s = make(M, K, N, M + K + N)
+        res = torch.randn(M, N, generator=torch.Generator().manual_seed(M)).half()
+        xd, pd, sd, rd = x.to(gpu), p.to(gpu), s.to(gpu), res.to(gpu)
+        ref = O.dequant_matmul(x.numpy(), u.numpy(), s.numpy(), np.float32)
+        print(f"pair split {cfg}: M={M} K={K} N={N}", flush=True)
+        for rep in range(2):
+            assert_close(gemm(xd, pd, sd, M, N, K).cpu().numpy(), ref, what=f"{cfg} plain M={M} K={K} N={N} rep {rep}")
+            got = fused(xd, pd, sd, M, N, K, 1, rd).cpu().numpy()
+            assert_close(got, O.residual_add(ref.astype(np.float16), res.numpy()), rtol=1e-2, atol=2e-3,
+                         what=f"{cfg} residual M={M} K={K} N={N} rep {rep}")
+    # not for the RMSnorm prologue or the SwiGLU epilogue: the table's choice runs
+    assert small_m_shape(8, 4096, 4096, 0, True)[3] == 1 and small_m_shape(8, 4096, 4096, 2, False)[3] == 1
+
 
 LARGE_M_TILES = ["8,4", "4,5", "4,4", "4,2", "2,2"]   # m-tiles, n-tiles per wavefront
 

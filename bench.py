@@ -85,7 +85,93 @@ def bench_lib():
     vp, sz = ctypes.c_void_p, ctypes.c_size_t
     h.eet_hbm_stream_probe.restype = ctypes.c_int
     h.eet_hbm_stream_probe.argtypes = [vp, sz, ctypes.c_int, vp, sz, vp]
+    i, f = ctypes.c_int, ctypes.c_float
+    h.eet_timeline_gemm_w8a16_fused.restype = i      # eet_gemm_w8a16_fused with clock readings in the kernel
+    h.eet_timeline_gemm_w8a16_fused.argtypes = [vp, vp, vp, vp, i, i, i, i, vp, vp, f, vp, sz, vp]
+    h.eet_timeline_begin.restype = i
+    h.eet_timeline_begin.argtypes = [i]
+    h.eet_timeline_launches.restype = i
+    h.eet_timeline_read.restype = i
+    h.eet_timeline_read.argtypes = [i, vp]
     return h
+
+
+def launch_timeline(torch, lib, weights, acts, outs, M):
+    """Where the time of a launch goes, read inside the kernel: the GEMM pass through the bench-only build of the
+    same source (eet_timeline_gemm_w8a16_fused), whose workgroups read the 100 MHz wall clock at entry, after their
+    first multiplied batch, at the end of the k loop, after issuing their stores and after the stores are
+    acknowledged.  Two passes are recorded; the second is analysed, by launch kind."""
+    import ctypes
+    import numpy as np
+    B = bench_lib()
+    st = torch.cuda.current_stream().cuda_stream
+    ws_need = max([lib.eet_gemm_w8a16_workspace(M, w.shape[1], w.shape[0], epi)
+                   for layer in weights for name, (w, s, epi) in layer.items() if name not in RMS_LAUNCHES] + [0])
+    ws = torch.zeros(max(ws_need // 4, 1), dtype=torch.float32, device=outs["gamma"].device)
+    calls, kinds = [], []
+    for layer in weights:
+        for name, (w, s, epi) in layer.items():
+            K, N = w.shape
+            n_out = N // 2 if epi == EPI_SWIGLU else N
+            res = outs["residual"].data_ptr() if epi == EPI_RESIDUAL else None
+            gam = outs["gamma"].data_ptr() if name in RMS_LAUNCHES else None
+            calls.append((acts[K].data_ptr(), w.data_ptr(), s.data_ptr(), outs[n_out].data_ptr(), M, N, K, epi, res, gam, 1e-6,
+                          None if gam or not ws_need else ws.data_ptr(), 0 if gam or not ws_need else ws.numel() * 4, st))
+            kinds.append(name)
+    n = len(calls)
+    if B.eet_timeline_begin(2 * n):
+        raise RuntimeError("eet_timeline_begin failed")
+    torch.cuda.synchronize()
+    for _ in range(2):
+        for c in calls:
+            if B.eet_timeline_gemm_w8a16_fused(*c):
+                raise RuntimeError(lib.eet_last_error().decode())
+    torch.cuda.synchronize()
+    if B.eet_timeline_launches() != 2 * n:
+        return {"error": f"{B.eet_timeline_launches()} launches recorded, {2 * n} made"}
+    buf = np.zeros(1024 * 8, dtype=np.uint64)
+    stamps = []
+    for l in range(n - 1, 2 * n):          # the last launch of the first pass, then the second pass
+        wgs = B.eet_timeline_read(l, buf.ctypes.data_as(ctypes.c_void_p))
+        if wgs <= 0:
+            return {"error": f"eet_timeline_read({l}) returned {wgs}"}
+        t = buf[: wgs * 8].reshape(wgs, 8).astype(np.int64)
+        stamps.append(t[t[:, 0] > 0])
+    out = {}
+    for kind in dict.fromkeys(kinds):
+        rows = []
+        for i in range(1, n):              # launch i of the second pass; i - 1 is its predecessor (stamps[0] = last of pass 1)
+            if kinds[i] != kind:
+                continue
+            prev, cur, nxt = stamps[i], stamps[i + 1], stamps[i + 2] if i + 2 < len(stamps) else None
+            t0 = cur[:, 0].min()
+            has1 = cur[:, 1] > 0
+            rows.append([
+                (nxt[:, 0].min() - t0) if nxt is not None else np.nan,      # period: entry to the next launch's entry
+                t0 - prev[:, 4].max(),                                      # last acknowledged store of the predecessor -> first entry
+                cur[:, 0].max() - t0,                                       # entry spread over the workgroups
+                (cur[has1, 1] - cur[has1, 0]).mean() if has1.any() else np.nan,   # entry -> first batch multiplied
+                (cur[:, 2] - t0).min(), (cur[:, 2] - t0).mean(), (cur[:, 2] - t0).max(),   # end of k loop after first entry
+                (cur[:, 3] - cur[:, 2]).mean(),                             # reduction + epilogue until the stores are issued
+                (cur[:, 4] - cur[:, 3]).mean(),                             # stores acknowledged
+                cur[:, 4].max() - t0,                                       # first entry -> last acknowledged store
+                (cur[:, 5] - cur[:, 6]).mean(),                             # first wavefront out of the k loop -> all out (barrier passed)
+                (cur[:, 5] - cur[:, 7]).mean(),                             # mean wavefront out of the k loop -> all out
+                (cur[:, 3] - cur[:, 5]).mean(),                             # barrier passed -> stores issued (the arithmetic of the epilogue)
+                (cur[:, 5] - t0).max()])                                    # the last workgroup's barrier after the first entry
+        a = np.nanmean(np.array(rows, dtype=np.float64), axis=0) / 100.0    # 100 MHz clock -> microseconds
+        out[kind] = {"launches": len(rows), "period_us": round(a[0], 2), "idle_before_first_entry_us": round(a[1], 2),
+                     "entry_spread_us": round(a[2], 2), "entry_to_first_batch_multiplied_us": round(a[3], 2),
+                     "k_loop_end_after_first_entry_us": {"first": round(a[4], 2), "mean": round(a[5], 2), "last": round(a[6], 2)},
+                     "reduce_and_epilogue_us": round(a[7], 2), "store_acknowledge_us": round(a[8], 2),
+                     "first_entry_to_last_acknowledge_us": round(a[9], 2),
+                     "wait_for_the_slowest_wavefront_us": {"from_the_first_wavefront_out": round(a[10], 2), "from_the_mean_wavefront_out": round(a[11], 2)},
+                     "epilogue_after_the_barrier_us": round(a[12], 2), "last_workgroup_barrier_after_first_entry_us": round(a[13], 2)}
+    out["what"] = ("clock readings inside the small-M kernel (bench-only build with -DEET_TIMELINE of the same source; thread 0 of "
+                   "each workgroup, 100 MHz wall clock), second of two recorded passes, mean over the launches of a kind; "
+                   "the instrumented kernel waits for its stores before its last reading, which the shipped one leaves to the "
+                   "end of the kernel")
+    return out
 
 
 def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup, probe=False, probe_grid_scale=1, chained=False):
@@ -595,6 +681,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the M = 1..32 sweep")
     ap.add_argument("--no-chain", action="store_true", help="skip the chained-launch form of the GEMM pass")
+    ap.add_argument("--no-timeline", action="store_true", help="skip the in-kernel clock readings of the GEMM pass")
     ap.add_argument("--no-baichuan", action="store_true",
                     help="skip benchmark configuration 5: Baichuan-13B-shaped decoder (40 layers, ALiBi), batch 32, "
                          "prompt 2048, 256 greedy tokens (needs ~85 GB of HBM and about a minute)")
@@ -695,6 +782,9 @@ def main():
                          "queue barrier (hipExtAnyOrderLaunch), requests its first weight batches and then waits in the "
                          "kernel (bounded) for the completion counter of the launch before it")
         result["chained_pass"] = chain
+
+    if not args.no_timeline:
+        result["launch_timeline"] = launch_timeline(torch, L, fused, acts, outs, M)
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(3)

@@ -24,6 +24,18 @@
 // applied once to the fp32 sum (the reference multiplies every weight by the
 // scale in fp16 first, mma_tensorop_dequantizer.h:258-275 -- this is strictly
 // more accurate and inside the 1e-2 / 1e-3 tolerance against fp32).
+//
+// Built a second time with -DEET_TIMELINE into the bench-only library: the same kernels with five
+// clock readings per workgroup (entry, first batch multiplied, k loop done, stores issued, stores
+// acknowledged), under entry-point names of their own, so that the measurement harness can say where the
+// time of a launch goes.  Nothing of it is compiled into the operator library.
+#if defined(EET_TIMELINE)
+#define eet_gemm_w8a16 eet_timeline_gemm_w8a16
+#define eet_gemm_w8a16_fused eet_timeline_gemm_w8a16_fused
+#define eet_gemm_w8a16_chained eet_timeline_gemm_w8a16_chained
+#define eet_gemm_w8a16_small_m_shape eet_timeline_gemm_w8a16_small_m_shape
+#define eet_gemm_w8a16_workspace eet_timeline_gemm_w8a16_workspace
+#endif
 #include <hip/hip_runtime.h>
 
 #include <hip/hip_ext.h>
@@ -33,6 +45,35 @@
 #include "tuning.h"
 
 using namespace eet;
+
+#if defined(EET_TIMELINE)
+#define EET_TL_PARAM , unsigned long long *tl
+#define EET_TL_ARG , timeline_next(grid_of_launch)
+#define EET_TL_NONE , nullptr
+#define EET_TL_STAMP(i)                                      \
+    do {                                                     \
+        if (tl != nullptr && threadIdx.x == 0)               \
+            tl_t[i] = wall_clock64();                        \
+    } while (0)
+namespace {
+constexpr int kTlStamps = 8, kTlMaxWgs = 1024;
+unsigned long long *g_tl_buf = nullptr;   // [launch][kTlMaxWgs][kTlStamps], device memory
+int g_tl_cap = 0, g_tl_n = 0;
+int g_tl_grid[4096];
+unsigned long long *timeline_next(int workgroups)
+{
+    if (g_tl_buf == nullptr || g_tl_n >= g_tl_cap || g_tl_n >= 4096 || workgroups > kTlMaxWgs)
+        return nullptr;
+    g_tl_grid[g_tl_n] = workgroups;
+    return g_tl_buf + (size_t)(g_tl_n++) * kTlMaxWgs * kTlStamps;
+}
+}  // namespace
+#else
+#define EET_TL_PARAM
+#define EET_TL_ARG
+#define EET_TL_NONE
+#define EET_TL_STAMP(i) do { } while (0)
+#endif
 
 namespace {
 
@@ -217,13 +258,25 @@ template <int NT, int RG, int WAVES, int U, bool RMS, int MODE>
 __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
     _Float16 *__restrict__ C, int M, int N, int K, const _Float16 *__restrict__ residual, int epi,
-    const _Float16 *__restrict__ rms_gamma, float rms_eps, eet::ChainLink link, PairArgs pair)
+    const _Float16 *__restrict__ rms_gamma, float rms_eps, eet::ChainLink link, PairArgs pair EET_TL_PARAM)
 {
     constexpr bool CHAIN = MODE == kChained, PAIR = MODE == kPair2 || MODE == kPair4;
     constexpr int KS = PAIR ? MODE : 1;
     static_assert(!PAIR || (!RMS && NT * ((RG + 1) / 2) <= kPairTiles), "k split: no RMSnorm prologue, at most 10 tiles");
 #if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
     constexpr int MT = (RG + 1) / 2;
+#if defined(EET_TIMELINE)
+    unsigned long long tl_t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    __shared__ unsigned long long tl_wave_end[WAVES];
+    auto tl_flush = [&]() {
+        if (tl != nullptr && threadIdx.x == 0) {
+            unsigned long long *q = tl + (size_t)(blockIdx.y * gridDim.x + blockIdx.x) * kTlStamps;
+            for (int i = 0; i < 8; ++i)
+                q[i] = tl_t[i];
+        }
+    };
+#endif
+    EET_TL_STAMP(0);
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: feeds scalar offsets
     const int g = lane >> 4, j = lane & 15;
@@ -374,6 +427,10 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
             for (; i + 2 <= nbatch; i += 2) {
                 load_batch<NT, RG, WAVES, U, RMS>(b1, wrsrc, wtile, lane, abase, gbase, kt + STEP, true);
                 mma_batch<NT, RG, U, RMS>(b0, acc, slab, lane, ss);
+#if defined(EET_TIMELINE)
+                if (i == 0)
+                    EET_TL_STAMP(1);
+#endif
                 load_batch<NT, RG, WAVES, U, RMS>(b0, wrsrc, wtile, lane, abase, gbase, kt + 2 * STEP, i + 2 < nbatch);
                 mma_batch<NT, RG, U, RMS>(b1, acc, slab, lane, ss);
                 kt += 2 * STEP;
@@ -390,6 +447,11 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         }
     }
 
+    EET_TL_STAMP(2);
+#if defined(EET_TIMELINE)
+    if (tl != nullptr && (threadIdx.x & 63) == 0)
+        tl_wave_end[threadIdx.x >> 6] = wall_clock64();   // every wavefront's end of the k loop
+#endif
     // RMSnorm prologue: each wavefront's share of sum(x^2) per row.  Lanes
     // 8*q .. 8*q+7 hold pieces of row 8*r + q.
     __shared__ float rowss[WAVES][RG * 8];
@@ -416,6 +478,18 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         for (int mt = 0; mt < MT; ++mt)
             red[(wave * NT * MT + t * MT + mt) * 64 + lane] = acc[t][mt];
     __syncthreads();
+#if defined(EET_TIMELINE)
+    EET_TL_STAMP(5);   // all wavefronts have left the k loop and written their partial sums
+    if (tl != nullptr && threadIdx.x == 0) {
+        unsigned long long lo = ~0ull, sum = 0;
+        for (int w = 0; w < WAVES; ++w) {
+            lo = tl_wave_end[w] < lo ? tl_wave_end[w] : lo;
+            sum += tl_wave_end[w] - tl_t[0];
+        }
+        tl_t[6] = lo;                    // the first wavefront to finish its k loop
+        tl_t[7] = tl_t[0] + sum / WAVES; // the mean over the wavefronts
+    }
+#endif
     auto tile_sum = [&](int tile) {
         floatx4 s = red[tile * 64 + lane];
 #pragma unroll
@@ -452,8 +526,14 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         if (threadIdx.x == 0)
             ticket = __hip_atomic_fetch_add(pair.tickets + blockIdx.x * 16, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
-        if (ticket != KS - 1)
+        if (ticket != KS - 1) {
+#if defined(EET_TIMELINE)
+            EET_TL_STAMP(3);
+            EET_TL_STAMP(4);
+            tl_flush();
+#endif
             return;   // the last arrival will find these sums and finish
+        }
         if (threadIdx.x == 0)   // ready for the next launch on this workspace
             __hip_atomic_store(pair.tickets + blockIdx.x * 16, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         i2 = 0;
@@ -513,6 +593,12 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     }
     if constexpr (CHAIN)
         eet::chain_signal(link);
+#if defined(EET_TIMELINE)
+    EET_TL_STAMP(3);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    EET_TL_STAMP(4);
+    tl_flush();
+#endif
 #endif
 }
 
@@ -526,8 +612,9 @@ int launch_small_m(const GemmArgs &a)
 {
     const int ntiles = a.N / 16;
     dim3 grid((ntiles + NT - 1) / NT), block(WAVES * 64);
+    [[maybe_unused]] const int grid_of_launch = (int)grid.x;
     hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U, RMS, kPlain>), grid, block, 0, a.st, a.A, a.Wp, a.scale,
-                       a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, eet::ChainLink{}, PairArgs{});
+                       a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, eet::ChainLink{}, PairArgs{} EET_TL_ARG);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
@@ -557,9 +644,10 @@ int launch_small_m_pair(const GemmArgs &a)
     PairArgs pa;
     pa.tickets = static_cast<unsigned *>(a.ws);
     pa.sums = reinterpret_cast<floatx4 *>(static_cast<char *>(a.ws) + kSplitTicketBytes);
+    [[maybe_unused]] const int grid_of_launch = groups * KS;
     hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U, false, KS>), dim3(groups, KS), dim3(WAVES * 64), 0, a.st,
                        a.A, a.Wp, a.scale, a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps,
-                       eet::ChainLink{}, pa);
+                       eet::ChainLink{}, pa EET_TL_ARG);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
@@ -578,10 +666,10 @@ int launch_small_m_chained(const GemmArgs &a)
     auto kern = w8a16_small_m_kernel<NT, RG, WAVES, U, RMS, kChained>;
     if (any_order)
         hipExtLaunchKernelGGL(kern, grid, block, 0, a.st, nullptr, nullptr, hipExtAnyOrderLaunch, a.A, a.Wp, a.scale,
-                              a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, link, PairArgs{});
+                              a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, link, PairArgs{} EET_TL_NONE);
     else
         hipLaunchKernelGGL(kern, grid, block, 0, a.st, a.A, a.Wp, a.scale, a.C, a.M, a.N, a.K, a.residual, a.epi,
-                           a.rms_gamma, a.rms_eps, link, PairArgs{});
+                           a.rms_gamma, a.rms_eps, link, PairArgs{} EET_TL_NONE);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
@@ -920,3 +1008,39 @@ extern "C" int eet_gemm_w8a16_chained(const void *A, const void *Wpacked, const 
     return gemm_fused("eet_gemm_w8a16_chained", A, Wpacked, scale, C, M, N, K, epilogue, residual, rms_gamma, rms_eps,
                       nullptr, 0, chain, stream);
 }
+
+#if defined(EET_TIMELINE)
+// Bench-only: recording starts with a device buffer for `launches` launches; every small-M launch made through the
+// eet_timeline_* entry points from then on fills the next slot.  eet_timeline_read synchronises the device, copies
+// slot `launch` ([workgroup][8] clock readings of the 100 MHz wall clock: entry, first batch multiplied, k loop
+// done, stores issued, stores acknowledged) and returns the workgroup count of that launch, or a negative value.
+extern "C" int eet_timeline_begin(int launches)
+{
+    if (g_tl_buf != nullptr && g_tl_cap < launches) {
+        (void)hipFree(g_tl_buf);
+        g_tl_buf = nullptr;
+    }
+    if (g_tl_buf == nullptr) {
+        EET_HIP_CHECK(hipMalloc(&g_tl_buf, (size_t)launches * kTlMaxWgs * kTlStamps * sizeof(unsigned long long)));
+        g_tl_cap = launches;
+    }
+    EET_HIP_CHECK(hipMemset(g_tl_buf, 0, (size_t)g_tl_cap * kTlMaxWgs * kTlStamps * sizeof(unsigned long long)));
+    g_tl_n = 0;
+    return EET_OK;
+}
+
+extern "C" int eet_timeline_launches(void) { return g_tl_n; }
+
+extern "C" int eet_timeline_read(int launch, unsigned long long *host_dst)
+{
+    if (launch < 0 || launch >= g_tl_n || host_dst == nullptr)
+        return -1;
+    if (hipDeviceSynchronize() != hipSuccess)
+        return -2;
+    const int wgs = g_tl_grid[launch];
+    if (hipMemcpy(host_dst, g_tl_buf + (size_t)launch * kTlMaxWgs * kTlStamps, (size_t)wgs * kTlStamps * sizeof(unsigned long long),
+                  hipMemcpyDeviceToHost) != hipSuccess)
+        return -2;
+    return wgs;
+}
+#endif

@@ -85,6 +85,8 @@ def bench_lib():
     vp, sz = ctypes.c_void_p, ctypes.c_size_t
     h.eet_hbm_stream_probe.restype = ctypes.c_int
     h.eet_hbm_stream_probe.argtypes = [vp, sz, ctypes.c_int, vp, sz, vp]
+    h.eet_hbm_stream_probe_ring.restype = ctypes.c_int
+    h.eet_hbm_stream_probe_ring.argtypes = [vp, sz, ctypes.c_int, vp, sz, vp]
     i, f = ctypes.c_int, ctypes.c_float
     h.eet_timeline_gemm_w8a16_fused.restype = i      # eet_gemm_w8a16_fused with clock readings in the kernel
     h.eet_timeline_gemm_w8a16_fused.argtypes = [vp, vp, vp, vp, i, i, i, i, vp, vp, f, vp, sz, vp]
@@ -174,7 +176,8 @@ def launch_timeline(torch, lib, weights, acts, outs, M):
     return out
 
 
-def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup, probe=False, probe_grid_scale=1, chained=False):
+def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup, probe=False, probe_grid_scale=1, chained=False,
+                   probe_ring=False):
     """Returns seconds per step (one pass over all linears), measured with
     events on the stream the kernels are launched on.  Launches named in
     RMS_LAUNCHES carry the RMSnorm prologue, as in the decoder.  probe=True
@@ -214,12 +217,13 @@ def time_gemm_pass(torch, lib, weights, acts, outs, M, steps, warmup, probe=Fals
                 mode = 2
     elif probe:
         sink = outs["probe_sink"]
-        g = bench_lib().eet_hbm_stream_probe
+        g = bench_lib().eet_hbm_stream_probe_ring if probe_ring else bench_lib().eet_hbm_stream_probe
 
         def one_pass():
             for (a, w, s, c, m, n, k, epi, res, gam) in calls:
                 # the grid the GEMM uses for this shape: 256 workgroups, 688 for the merged gate|up matrix
-                rc = g(w, k * n, (688 if epi == EPI_SWIGLU else 256) * probe_grid_scale, sink.data_ptr(), sink.numel(), sp)
+                rc = g(w, k * n, (688 if epi == EPI_SWIGLU and not probe_ring else 256) * probe_grid_scale, sink.data_ptr(),
+                       sink.numel(), sp)
                 if rc:
                     raise RuntimeError("eet_hbm_stream_probe failed")
     else:
@@ -728,8 +732,10 @@ def main():
     per_launch_us = sec / launches * 1e6
     # the same chain of launches as pure reads of the same weight buffers: what the machine allows
     # (256 workgroups per launch, 688 for gate|up, and two and four times as many: the best of the three counts)
-    probe_sec = min(time_gemm_pass(torch, L, fused, acts, outs, M, max(3, args.steps // 2), 1, probe=True,
-                                   probe_grid_scale=sc)[0] for sc in (1, 2, 4))
+    probe_sec = min([time_gemm_pass(torch, L, fused, acts, outs, M, max(3, args.steps // 2), 1, probe=True,
+                                    probe_grid_scale=sc)[0] for sc in (1, 2, 4)] +
+                    [time_gemm_pass(torch, L, fused, acts, outs, M, max(3, args.steps // 2), 1, probe=True,
+                                    probe_grid_scale=sc, probe_ring=True)[0] for sc in (1, 2)])
     weight_bytes = sum(w.numel() for layer in fused for (w, _, _) in layer.values())
     ceiling_gbs = weight_bytes / probe_sec / 1e9
     traffic, traffic_file = recorded_traffic(M, args.layers)
@@ -757,8 +763,9 @@ def main():
                      "stream_ceiling": {"GB/s": round(ceiling_gbs, 1), "frac_of_peak": round(ceiling_gbs / HBM_PEAK_GBS, 4),
                                         "ms_per_step": round(probe_sec * 1e3, 4),
                                         "what": "the same 128 launches per step as read-only streams of the same weight "
-                                                "buffers (eet_hbm_stream_probe; 256 workgroups per launch, 688 for gate|up, also at "
-                                                "twice and four times as many, best of the three): the rate this machine "
+                                                "buffers (eet_hbm_stream_probe: two batches of four loads per lane in flight, 256 workgroups per launch, 688 "
+                                                "for gate|up, also twice and four times as many; eet_hbm_stream_probe_ring: a ring of four loads "
+                                                "per lane without a branch, 256 and 512 workgroups; the best of the five): the rate this machine "
                                                 "allows a chain of dependent launches of these sizes"},
                      "frac_of_stream_ceiling": round(step_bytes / sec / (weight_bytes / probe_sec), 4)},
         "host_wall_ms_per_step": round(wall * 1e3, 4),

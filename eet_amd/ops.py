@@ -230,12 +230,14 @@ RMS_FUSE_MAX_M = 32     # the RMSnorm prologue exists in the small-M kernel only
 
 def _k_split_ws(M, N, K, epilogue, device):
     """(pointer, bytes) of the small-M kernel's k-split workspace for this call, or (None, 0).  A buffer of its
-    own, zero when created (the arrival counters at its start must start at zero; every call leaves them so),
-    and one per stream: launches that share it must be ordered, and only the launches of one stream are."""
+    own, zero when created (the arrival counters at its start must start at zero; every call leaves them so).
+    One buffer per device, like every named workspace here (and like the reference's MManager buffers,
+    csrc/op/mmanager.hpp:141-205): the ops of a process are meant to run on one stream; launches on two
+    streams that can overlap in time must not share it."""
     need = lib().eet_gemm_w8a16_workspace(M, N, K, epilogue) if M <= RMS_FUSE_MAX_M else 0
     if not need:
         return None, 0
-    buf = workspaces.get(f"gemm_small_m_k_split@{_stream() or 0}", (need + 3) // 4, torch.float32, device, zero=True)
+    buf = workspaces.get("gemm_small_m_k_split", (need + 3) // 4, torch.float32, device, zero=True)
     return buf.data_ptr(), buf.numel() * 4
 
 

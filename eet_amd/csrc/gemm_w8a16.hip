@@ -942,6 +942,10 @@ extern "C" int eet_gemm_w8a16_small_m_shape(int M, int N, int K, int epilogue, i
     a.M = M, a.N = N, a.K = K, a.epi = epilogue;
     static const _Float16 kSomeGamma = 0;
     a.rms_gamma = rms_prologue ? &kSomeGamma : nullptr;   // only tested against null
+    // as for a call that hands over the workspace eet_gemm_w8a16_workspace asks for (never dereferenced here)
+    static const u32x4 kSomeWorkspace = {0, 0, 0, 0};
+    a.ws = const_cast<u32x4 *>(&kSomeWorkspace);
+    a.ws_bytes = ~size_t(0);
     const SmallMConfig cfg = resolve_small_m(a);
     *nt = cfg.nt, *waves = cfg.waves, *k_tiles_per_batch = cfg.u, *k_split = cfg.ksplit;
     return EET_OK;

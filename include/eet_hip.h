@@ -165,7 +165,8 @@ int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, 
 
 /* The launch shape the small-M kernel (1 <= M <= 32) runs a call with: n-tiles per
  * workgroup, wavefronts per workgroup, k-tiles per register batch, and how many
- * workgroups share a tile's k range (1, or 2 for the pair split) -- the tuning
+ * workgroups share a tile's k range (1, 2 or 4; what a call runs with when it hands
+ * over the workspace eet_gemm_w8a16_workspace asks for -- without it, 1) -- the tuning
  * override EET_GEMM_SMALL_M_CONFIG when a kernel of that shape exists for the
  * call, otherwise the table's choice.  For sweeps and for tests that must know
  * which variant ran.  The reference's counterpart is the CutlassGemmConfig its

@@ -186,6 +186,19 @@ def test_pair_split(gpu, tuning, cfg):
     assert small_m_shape(8, 4096, 4096, 0, True)[3] == 1 and small_m_shape(8, 4096, 4096, 2, False)[3] == 1
 
 
+def test_k_split_dispatch(gpu):
+    """What the table picks (no override) for a call that hands over the workspace: the k split for the O / down
+    launches of both decoders at the batch sizes where it measured faster, the plain launch elsewhere."""
+    assert small_m_shape(16, 4096, 4096, 1, False) == (2, 4, 2, 2)       # LLaMA O, M = 16
+    assert small_m_shape(32, 4096, 11008, 1, False) == (4, 8, 1, 4)      # LLaMA down, M = 32
+    assert small_m_shape(8, 4096, 4096, 1, False)[3] == 1                # M <= 8: not on the LLaMA shapes
+    assert small_m_shape(8, 5120, 5120, 1, False) == (5, 8, 1, 4)        # Baichuan O: 320 n-tiles as 64 groups x 4
+    assert small_m_shape(32, 5120, 5120, 1, False)[3] == 1               # ... but not at M = 32 with the short k range
+    assert small_m_shape(32, 5120, 13696, 1, False) == (5, 8, 1, 4)
+    assert small_m_shape(16, 12288, 4096, 0, True)[3] == 1               # never with the RMSnorm prologue
+    assert small_m_shape(16, 4112, 4096, 1, False)[3] == 1               # other channel counts keep the table's choice
+
+
 LARGE_M_TILES = ["8,4", "4,5", "4,4", "4,2", "2,2"]   # m-tiles, n-tiles per wavefront
 
 

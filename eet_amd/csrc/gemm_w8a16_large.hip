@@ -183,12 +183,18 @@ __global__ __launch_bounds__(64 * WNW) __attribute__((amdgpu_waves_per_eu(2))) v
             __builtin_amdgcn_sched_group_barrier(0x008, 2 * TN, 0);  // 2*TN MFMA
         }
         __builtin_amdgcn_sched_barrier(0);
-        // The DMA of tile kt+1 (issued two steps ago) must have landed before any
-        // wavefront reads it: everything older than the loads of the last two steps
-        // (2 x (kPerWave DMA + TN weight loads)), then the barrier.
+        // The DMA of tile kt+1 (issued two steps ago) must have landed before any wavefront reads it.  Accesses that
+        // touch memory complete in the order issued, register loads and copies into LDS alike; one whose lanes are ALL
+        // out of range (the row groups past M of a ragged block) completes at once, ahead of older copies (measured:
+        // a counted wait over such accesses let an older copy through).  So the count has to hold with every such
+        // access already gone.  Younger than that DMA are, among others, three weight batches (3 TN loads that always
+        // touch memory); once no more than kPerWave + TN accesses are outstanding (the ones this step issued), the
+        // complete ones include everything but the youngest kPerWave + TN <= 3 TN real ones, hence the DMA in
+        // question.  Costs under 0.5 % against allowing the loads of two steps to be outstanding, which only timing
+        // made safe on ragged blocks.
         // (A plain __syncthreads() would drain every outstanding load here: its
         // release fence waits for all DMA writes, including the ones just issued.)
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * (S::kPerWave + TN)) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(S::kPerWave + TN) : "memory");
     };
 
     // prologue: tiles 0..2 into stages 0..2, weights of tiles 0 and 1

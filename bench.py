@@ -732,15 +732,29 @@ def main():
     per_launch_us = sec / launches * 1e6
     # the same chain of launches as pure reads of the same weight buffers: what the machine allows
     # (256 workgroups per launch, 688 for gate|up, and two and four times as many: the best of the three counts)
-    probe_sec = min([time_gemm_pass(torch, L, fused, acts, outs, M, max(3, args.steps // 2), 1, probe=True,
-                                    probe_grid_scale=sc)[0] for sc in (1, 2, 4)] +
-                    [time_gemm_pass(torch, L, fused, acts, outs, M, max(3, args.steps // 2), 1, probe=True,
-                                    probe_grid_scale=sc, probe_ring=True)[0] for sc in (1, 2)])
     weight_bytes = sum(w.numel() for layer in fused for (w, _, _) in layer.values())
-    ceiling_gbs = weight_bytes / probe_sec / 1e9
+    try:
+        probe_sec = min([time_gemm_pass(torch, L, fused, acts, outs, M, max(3, args.steps // 2), 1, probe=True,
+                                        probe_grid_scale=sc)[0] for sc in (1, 2, 4)] +
+                        [time_gemm_pass(torch, L, fused, acts, outs, M, max(3, args.steps // 2), 1, probe=True,
+                                        probe_grid_scale=sc, probe_ring=True)[0] for sc in (1, 2)])
+        ceiling_gbs = weight_bytes / probe_sec / 1e9
+        probe_error = None
+    except (RuntimeError, OSError, AttributeError) as e:   # the measurement-only library is missing or stale: the headline stands without it
+        probe_sec, ceiling_gbs, probe_error = float("nan"), float("nan"), str(e)
     traffic, traffic_file = recorded_traffic(M, args.layers)
     traffic_source = (f"{traffic_file}: FETCH_SIZE + WRITE_SIZE of this command under rocprofv3 --pmc, recorded when that "
                       "file was committed; NOT measured in this run (counters need the profiler)") if traffic_file else None
+    if probe_error is None:
+        stream_ceiling = {"GB/s": round(ceiling_gbs, 1), "frac_of_peak": round(ceiling_gbs / HBM_PEAK_GBS, 4),
+                          "ms_per_step": round(probe_sec * 1e3, 4),
+                          "what": "the same 128 launches per step as read-only streams of the same weight "
+                                  "buffers (eet_hbm_stream_probe: two batches of four loads per lane in flight, 256 workgroups per launch, 688 "
+                                  "for gate|up, also twice and four times as many; eet_hbm_stream_probe_ring: a ring of four loads "
+                                  "per lane without a branch, 256 and 512 workgroups; the best of the five): the rate this machine "
+                                  "allows a chain of dependent launches of these sizes"}
+    else:
+        stream_ceiling = {"error": probe_error}
     result = {
         "metric": "int8 W-only GEMM HBM GB/s (% peak) at M=1..16; LLaMA-7B int8 decode tokens/s, 1 GPU",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -760,14 +774,8 @@ def main():
                      # HBM-side bytes per launch, from the committed rocprofv3 --pmc summary of this workload
                      # (FETCH_SIZE and WRITE_SIZE scaled by a copy kernel of known size); null if none matches
                      "traffic": traffic, "traffic_source": traffic_source,
-                     "stream_ceiling": {"GB/s": round(ceiling_gbs, 1), "frac_of_peak": round(ceiling_gbs / HBM_PEAK_GBS, 4),
-                                        "ms_per_step": round(probe_sec * 1e3, 4),
-                                        "what": "the same 128 launches per step as read-only streams of the same weight "
-                                                "buffers (eet_hbm_stream_probe: two batches of four loads per lane in flight, 256 workgroups per launch, 688 "
-                                                "for gate|up, also twice and four times as many; eet_hbm_stream_probe_ring: a ring of four loads "
-                                                "per lane without a branch, 256 and 512 workgroups; the best of the five): the rate this machine "
-                                                "allows a chain of dependent launches of these sizes"},
-                     "frac_of_stream_ceiling": round(step_bytes / sec / (weight_bytes / probe_sec), 4)},
+                     "stream_ceiling": stream_ceiling,
+                     "frac_of_stream_ceiling": round(step_bytes / sec / (weight_bytes / probe_sec), 4) if probe_error is None else None},
         "host_wall_ms_per_step": round(wall * 1e3, 4),
     }
 
@@ -791,7 +799,10 @@ def main():
         result["chained_pass"] = chain
 
     if not args.no_timeline:
-        result["launch_timeline"] = launch_timeline(torch, L, fused, acts, outs, M)
+        try:
+            result["launch_timeline"] = launch_timeline(torch, L, fused, acts, outs, M)
+        except (RuntimeError, OSError, AttributeError) as e:
+            result["launch_timeline"] = {"error": str(e)}
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(3)

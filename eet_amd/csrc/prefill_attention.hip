@@ -67,11 +67,35 @@ __device__ __forceinline__ float max_over_lane_groups(float v)
     return v;
 }
 
+// Which (batch, head) pair and query block a workgroup takes.  Workgroup i runs on XCD i % 8 and the XCDs have an
+// L2 each, so the workgroups that are resident on an XCD at one time should be the query blocks of FEW pairs: they
+// walk the same K and V rows at about the same time and fetch each of them once between them.  With `group` > 0
+// and a pair count divisible by 8, XCD x owns the pairs x, x + 8, ... in groups of `group`; inside a group the
+// longest (last) query block of every pair is handed out first, then the one before (the long blocks start first,
+// the short ones fill the tail, group after group).  group = 0: all pairs of the last query block first, then
+// those of the one before, over the whole launch (every resident workgroup then has a pair of its own, and a
+// prompt's K and V cross the fabric once per query block instead of once).
+__device__ __forceinline__ void prefill_block_of(int group, int *bh, int *qblock)
+{
+    const int pairs = gridDim.x, q_blocks = gridDim.y;
+    if (group <= 0 || pairs % 8 != 0) {
+        *bh = blockIdx.x;
+        *qblock = q_blocks - 1 - (int)blockIdx.y;
+        return;
+    }
+    const int lin = blockIdx.y * pairs + blockIdx.x;
+    const int xcd = lin % 8, q = lin / 8, per_xcd = pairs / 8;
+    const int gs = group * q_blocks, g = q / gs, r = q % gs;
+    const int gl = min(group, per_xcd - g * group);       // pairs of this group (the last may be smaller)
+    *bh = (g * group + r % gl) * 8 + xcd;
+    *qblock = q_blocks - 1 - r / gl;
+}
+
 template <int DH>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void prefill_attention_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_cache, const _Float16 *__restrict__ v_cache,
     _Float16 *__restrict__ ctx, const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, int H, int S,
-    int T_cap, float scale)
+    int T_cap, float scale, int group)
 {
 #if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
     constexpr int DC = DH / 32;            // 32-wide d chunks of the first product
@@ -84,10 +108,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 4, j = lane & 15;
-    // all (batch, head) pairs of the last (longest) query block are handed out first, then the one before, ...
-    const int bh = blockIdx.x, b = bh / H, h = bh % H;
-    const int q_blocks = (S + kBQ - 1) / kBQ;
-    const int q0 = (q_blocks - 1 - (int)blockIdx.y) * kBQ;
+    int bh, qblock;
+    prefill_block_of(group, &bh, &qblock);
+    const int b = bh / H, h = bh % H;
+    const int q0 = qblock * kBQ;
     const int padb = pad ? (int)min((int64_t)S, max((int64_t)0, pad[b])) : 0;
 
     const _Float16 *kbase = k_cache + (size_t)bh * T_cap * DH;
@@ -367,7 +391,7 @@ __global__ __launch_bounds__(64 * WAVES)
     __attribute__((amdgpu_waves_per_eu(STAGES == 2 ? 2 * WAVES / 4 : WAVES / 4, STAGES == 2 ? 2 * WAVES / 4 : WAVES / 4))) void prefill_attention_dh128_kernel(
     const _Float16 *__restrict__ q, const _Float16 *__restrict__ k_cache, const _Float16 *__restrict__ v_cache,
     _Float16 *__restrict__ ctx, const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, int H, int S,
-    int T_cap, float scale)
+    int T_cap, float scale, int group)
 {
 #if defined(__HIP_DEVICE_COMPILE__)  // buffer-resource builtins exist in the device pass only
     constexpr int DC = kD / 32, DT = kD / 16;
@@ -378,12 +402,12 @@ __global__ __launch_bounds__(64 * WAVES)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 4, j = lane & 15;
-    // Workgroups are handed out in index order: all (batch, head) pairs of the last query block first, then
-    // those of the one before, so the long blocks start first over the whole launch and the short ones fill
-    // the tail (with the block index running fastest the last CU to finish held up to a fifth of the launch).
-    const int bh = blockIdx.x, b = bh / H, h = bh % H;
-    const int q_blocks = (S + kBQ2 - 1) / kBQ2;
-    const int q0 = (q_blocks - 1 - (int)blockIdx.y) * kBQ2;
+    // Workgroups take (pair, query block) in the order of prefill_block_of: long blocks before short ones (with the
+    // block index running fastest the last CU to finish held up to a fifth of the launch), few pairs per XCD at a time.
+    int bh, qblock;
+    prefill_block_of(group, &bh, &qblock);
+    const int b = bh / H, h = bh % H;
+    const int q0 = qblock * kBQ2;
     const int padb = pad ? (int)min((int64_t)S, max((int64_t)0, pad[b])) : 0;
 
     const _Float16 *kbase = k_cache + (size_t)bh * T_cap * kD;
@@ -664,6 +688,23 @@ __global__ __launch_bounds__(64 * WAVES)
 #endif
 }
 
+// Pairs per XCD group (prefill_block_of): as many as fill the workgroup slots of an XCD with all their query
+// blocks, at least four (measured at B*H = 256 .. 1280, 512 .. 8192 tokens: 4 .. 16 pairs are within noise of one
+// another and 5-12 % ahead of the ungrouped order; one or two pairs lose to it, their long blocks idle too many CUs
+// while they finish).  A launch that fits the slots in one round keeps the ungrouped order: there the dispatcher
+// pairs workgroup i with workgroup i + 32 on a CU, and only that order makes it a long block with a short one.
+// The tuning key EET_PREFILL_GROUP forces a count, -1 the ungrouped order.
+int pairs_per_group(int slots_per_xcd, int q_blocks, int pairs)
+{
+    const int forced = eet::tuning().prefill_group;
+    if (forced != 0)
+        return forced < 0 ? 0 : forced;
+    if (q_blocks < 1 || pairs % 8 != 0 || (pairs / 8) * q_blocks <= slots_per_xcd)
+        return 0;
+    const int g = slots_per_xcd / q_blocks;
+    return g < 4 ? 4 : g;
+}
+
 int launch_dh128(const void *q, const void *kc, const void *vc, void *ctx, const void *alibi, const int64_t *pad, int B,
                  int H, int S, int T_cap, hipStream_t st)
 {
@@ -683,7 +724,8 @@ int launch_dh128(const void *q, const void *kc, const void *vc, void *ctx, const
                        dim3(B * H, (S + 16 * N_ * W_ - 1) / (16 * N_ * W_)), dim3(64 * W_), 0, st,                \
                        static_cast<const _Float16 *>(q), static_cast<const _Float16 *>(kc),                       \
                        static_cast<const _Float16 *>(vc), static_cast<_Float16 *>(ctx),                           \
-                       static_cast<const _Float16 *>(alibi), pad, H, S, T_cap, scale)
+                       static_cast<const _Float16 *>(alibi), pad, H, S, T_cap, scale,                             \
+                       pairs_per_group(32 * (shape == 1 ? 2 : 1), (S + 16 * N_ * W_ - 1) / (16 * N_ * W_), B * H))
     if (alibi != nullptr) {
         if (shape == 1)
             EET_PF_LAUNCH(true, 1, 8, 2);
@@ -708,7 +750,8 @@ int launch(const void *q, const void *kc, const void *vc, void *ctx, const void 
     dim3 grid(B * H, (S + kBQ - 1) / kBQ);
     hipLaunchKernelGGL((prefill_attention_kernel<DH>), grid, dim3(kThreads), 0, st, static_cast<const _Float16 *>(q),
                        static_cast<const _Float16 *>(kc), static_cast<const _Float16 *>(vc),
-                       static_cast<_Float16 *>(ctx), static_cast<const _Float16 *>(alibi), pad, H, S, T_cap, scale);
+                       static_cast<_Float16 *>(ctx), static_cast<const _Float16 *>(alibi), pad, H, S, T_cap, scale,
+                       pairs_per_group(64, (int)grid.y, B * H));
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }

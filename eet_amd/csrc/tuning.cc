@@ -48,6 +48,8 @@ int apply(const char *name, const char *value)
         slot = &t.prefill_legacy;
     else if (std::strcmp(name, "EET_PREFILL_SHAPE") == 0)
         slot = &t.prefill_shape;
+    else if (std::strcmp(name, "EET_PREFILL_GROUP") == 0)
+        slot = &t.prefill_group;
     else if (std::strcmp(name, "EET_CHAIN_SLEEP") == 0)
         slot = &t.chain_sleep;
     else if (std::strcmp(name, "EET_CHAIN_SPIN_LIMIT") == 0) {
@@ -68,7 +70,7 @@ struct EnvInit {
         if (on == nullptr || std::strcmp(on, "1") != 0)
             return;
         for (const char *name : {"EET_GEMM_SMALL_M_CONFIG", "EET_GEMM_LARGE_M_TILE", "EET_MMHA_NSPLIT",
-                                 "EET_MMHA_THREADS", "EET_MMHA_UNROLL", "EET_PREFILL_LEGACY", "EET_PREFILL_SHAPE",
+                                 "EET_MMHA_THREADS", "EET_MMHA_UNROLL", "EET_PREFILL_LEGACY", "EET_PREFILL_SHAPE", "EET_PREFILL_GROUP",
                                  "EET_CHAIN_SLEEP", "EET_CHAIN_SPIN_LIMIT"})
             if (const char *v = std::getenv(name))
                 if (apply(name, v) != EET_OK)

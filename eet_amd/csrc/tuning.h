@@ -20,6 +20,7 @@ struct Tuning {
     // EET_PREFILL_LEGACY = 1: head size 128 takes the register-staged prefill attention kernel
     int prefill_legacy = 0;
     int prefill_shape = 0;   // 1, 2: launch shape of the head-size-128 prefill attention kernel; 0 = by prompt length
+    int prefill_group = 0;   // EET_PREFILL_GROUP: (batch, head) pairs per XCD group of the prefill attention order; -1: ungrouped
     // EET_CHAIN_SPIN_LIMIT: polls before a chained wait gives up (-1: the default, 65536; 0 gives up at once);
     // EET_CHAIN_SLEEP: s_sleep(8) repetitions between two polls (0: the default, 1)
     int chain_spin_limit = -1, chain_sleep = 0;

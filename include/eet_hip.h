@@ -53,6 +53,8 @@ int eet_packed_layout_version(void);
  *   EET_MMHA_NSPLIT / EET_MMHA_THREADS / EET_MMHA_UNROLL "n"
  *   EET_PREFILL_LEGACY "1" (register-staged prefill attention at head size 128)
  *   EET_PREFILL_SHAPE "1" | "2" (launch shape of the head-size-128 prefill kernel)
+ *   EET_PREFILL_GROUP "n" ((batch, head) pairs whose query blocks an XCD works on together in prefill
+ *                         attention; "-1": every pair of a query block before the next block)
  *   EET_CHAIN_SPIN_LIMIT "n" / EET_CHAIN_SLEEP "n" (bounded wait of a chained launch)
  * An override naming a kernel variant that does not exist is ignored.  The same
  * keys are read from the environment once, at load, when EET_HIP_TUNING=1; no

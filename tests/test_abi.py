@@ -154,7 +154,8 @@ def test_tuning_keys():
     for name, value in [("EET_GEMM_SMALL_M_CONFIG", "2,8,1"), ("EET_GEMM_SMALL_M_CONFIG", "2,8,1,2"),
                         ("EET_CHAIN_SPIN_LIMIT", "0"), ("EET_CHAIN_SLEEP", "4"), ("EET_GEMM_LARGE_M_TILE", "4,4"),
                         ("EET_GEMM_LARGE_M_TILE", "2,2,4"), ("EET_MMHA_NSPLIT", "2"), ("EET_MMHA_THREADS", "256"),
-                        ("EET_MMHA_UNROLL", "4"), ("EET_PREFILL_LEGACY", "1"), ("EET_PREFILL_SHAPE", "2")]:
+                        ("EET_MMHA_UNROLL", "4"), ("EET_PREFILL_LEGACY", "1"), ("EET_PREFILL_SHAPE", "2"),
+                        ("EET_PREFILL_GROUP", "4"), ("EET_PREFILL_GROUP", "-1")]:
         assert L.eet_set_tuning(name.encode(), value.encode()) == 0, L.eet_last_error()
         assert L.eet_set_tuning(name.encode(), None) == 0
     assert L.eet_set_tuning(b"EET_GEMM_SMALL_M_CONFIG", b"2,8") != 0

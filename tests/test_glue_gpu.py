@@ -151,6 +151,26 @@ def test_prefill_attention_launch_shapes_dh128(gpu, tuning, shape, S, use_pad, u
     test_prefill_attention(gpu, 2, 2, S, 128, use_pad, use_alibi)
 
 
+@pytest.mark.parametrize("group", [-1, 1, 2, 5])
+@pytest.mark.parametrize("B,H,S,dh", [(4, 6, 700, 128), (2, 8, 1600, 128), (4, 4, 300, 64)])
+def test_prefill_attention_workgroup_order(gpu, tuning, group, B, H, S, dh):
+    """Which (batch, head) pair and query block a workgroup takes is a permutation chosen for the XCDs' L2
+    caches (pairs in groups per XCD, long query blocks first); every forced group size -- also one that does not
+    divide the pairs of an XCD, and the ungrouped order -- must cover every (pair, block) exactly once: the
+    context buffer starts as NaN and is held to the oracle everywhere."""
+    tuning("EET_PREFILL_GROUP", group)
+    g = torch.Generator().manual_seed(S + group)
+    q, k, v = [torch.randn(B, H, S, dh, generator=g).half() for _ in range(3)]
+    want = O.prefill_attention(q.numpy(), k.numpy(), v.numpy(), None, None)
+    ctx = torch.full((B, S, H * dh), float("nan"), dtype=torch.float16, device=gpu)
+    qd, kcd, vcd = q.to(gpu), k.to(gpu).contiguous(), v.to(gpu).contiguous()
+    check(lib().eet_prefill_attention(qd.data_ptr(), kcd.data_ptr(), vcd.data_ptr(), ctx.data_ptr(), None, None,
+                                      B, H, S, dh, S, stream()))
+    got = ctx.cpu().numpy()
+    assert not np.isnan(got).any(), "a (pair, query block) was left out"
+    assert_close(got, want, what=f"prefill ctx, group {group}")
+
+
 @pytest.mark.parametrize("S,use_alibi", [(300, False), (130, True)])
 def test_prefill_attention_register_staged_kernel_dh128(gpu, tuning, S, use_alibi):
     """Head size 128 normally takes the DMA kernel; the register-staged one (the path of the other head

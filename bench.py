@@ -62,6 +62,7 @@ def make_weights(torch, eet, dev, layers, hidden, d_ff, seed):
 
 
 RMS_LAUNCHES = ("rmsnorm+qkv", "rmsnorm+gate|up+swiglu")     # the launches that carry the RMSnorm prologue
+TIMELINE_READINGS = 24   # per workgroup in the bench-only build: 8 of the workgroup, then one per wavefront (up to 16)
 
 
 def fused_launch_weights(eet_ops, weights):
@@ -131,13 +132,13 @@ def launch_timeline(torch, lib, weights, acts, outs, M):
     torch.cuda.synchronize()
     if B.eet_timeline_launches() != 2 * n:
         return {"error": f"{B.eet_timeline_launches()} launches recorded, {2 * n} made"}
-    buf = np.zeros(1024 * 8, dtype=np.uint64)
+    buf = np.zeros(1024 * TIMELINE_READINGS, dtype=np.uint64)
     stamps = []
     for l in range(n - 1, 2 * n):          # the last launch of the first pass, then the second pass
         wgs = B.eet_timeline_read(l, buf.ctypes.data_as(ctypes.c_void_p))
         if wgs <= 0:
             return {"error": f"eet_timeline_read({l}) returned {wgs}"}
-        t = buf[: wgs * 8].reshape(wgs, 8).astype(np.int64)
+        t = buf[: wgs * TIMELINE_READINGS].reshape(wgs, TIMELINE_READINGS)[:, :8].astype(np.int64)
         stamps.append(t[t[:, 0] > 0])
     out = {}
     for kind in dict.fromkeys(kinds):

@@ -56,7 +56,7 @@ using namespace eet;
             tl_t[i] = wall_clock64();                        \
     } while (0)
 namespace {
-constexpr int kTlStamps = 8, kTlMaxWgs = 1024;
+constexpr int kTlStamps = 24, kTlMaxWgs = 1024;   // 8 readings of the workgroup, then one per wavefront
 unsigned long long *g_tl_buf = nullptr;   // [launch][kTlMaxWgs][kTlStamps], device memory
 int g_tl_cap = 0, g_tl_n = 0;
 int g_tl_grid[4096];
@@ -268,6 +268,7 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
 #if defined(EET_TIMELINE)
     unsigned long long tl_t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     __shared__ unsigned long long tl_wave_end[WAVES];
+    __shared__ unsigned tl_wave_hw[WAVES];
     auto tl_flush = [&]() {
         if (tl != nullptr && threadIdx.x == 0) {
             unsigned long long *q = tl + (size_t)(blockIdx.y * gridDim.x + blockIdx.x) * kTlStamps;
@@ -449,8 +450,10 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
 
     EET_TL_STAMP(2);
 #if defined(EET_TIMELINE)
-    if (tl != nullptr && (threadIdx.x & 63) == 0)
+    if (tl != nullptr && (threadIdx.x & 63) == 0) {
         tl_wave_end[threadIdx.x >> 6] = wall_clock64();   // every wavefront's end of the k loop
+        tl_wave_hw[threadIdx.x >> 6] = __builtin_amdgcn_s_getreg(63492) & 0xffff;
+    }
 #endif
     // RMSnorm prologue: each wavefront's share of sum(x^2) per row.  Lanes
     // 8*q .. 8*q+7 hold pieces of row 8*r + q.
@@ -488,6 +491,11 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         }
         tl_t[6] = lo;                    // the first wavefront to finish its k loop
         tl_t[7] = tl_t[0] + sum / WAVES; // the mean over the wavefronts
+        // per wavefront: the end of its k loop after the workgroup's entry (low 32 bits) and where it ran
+        // (HW_ID bits 0-15 above them: wave slot, SIMD, CU, shader array and engine)
+        unsigned long long *q = tl + (size_t)(blockIdx.y * gridDim.x + blockIdx.x) * kTlStamps + 8;
+        for (int w = 0; w < WAVES; ++w)
+            q[w] = ((tl_wave_end[w] - tl_t[0]) & 0xffffffffull) | ((unsigned long long)tl_wave_hw[w] << 32);
     }
 #endif
     auto tile_sum = [&](int tile) {
@@ -536,16 +544,21 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
         }
         if (threadIdx.x == 0)   // ready for the next launch on this workspace
             __hip_atomic_store(pair.tickets + blockIdx.x * 16, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // The shares are added in the order of the k range, whichever workgroup came last: the rounding of
+        // the sum, and with it the result, does not depend on the order of arrival.
         i2 = 0;
         for (int unit = wave; unit < units; unit += WAVES, ++i2) {
+            floatx4 part[KS];
 #pragma unroll
-            for (int o = 1; o < KS; ++o) {
-                const unsigned share = (blockIdx.y + o) % KS;
-                const u32x4 v = __builtin_bit_cast(
-                    u32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                               prs, (unsigned)(((share * kTiles + unit) * 64 + lane) * 16), 0, kAgentScope));
-                whole[i2] += __builtin_bit_cast(floatx4, v);
-            }
+            for (int o = 0; o < KS; ++o)
+                part[o] = __builtin_bit_cast(
+                    floatx4, __builtin_amdgcn_raw_buffer_load_b128(
+                                 prs, (unsigned)(((o * kTiles + unit) * 64 + lane) * 16), 0, kAgentScope));
+            floatx4 tot = blockIdx.y == 0 ? whole[i2] : part[0];
+#pragma unroll
+            for (int o = 1; o < KS; ++o)
+                tot += (int)blockIdx.y == o ? whole[i2] : part[o];
+            whole[i2] = tot;
         }
     }
     int idx = 0;
@@ -1016,7 +1029,7 @@ extern "C" int eet_gemm_w8a16_chained(const void *A, const void *Wpacked, const 
 #if defined(EET_TIMELINE)
 // Bench-only: recording starts with a device buffer for `launches` launches; every small-M launch made through the
 // eet_timeline_* entry points from then on fills the next slot.  eet_timeline_read synchronises the device, copies
-// slot `launch` ([workgroup][8] clock readings of the 100 MHz wall clock: entry, first batch multiplied, k loop
+// slot `launch` ([workgroup][24]: 8 clock readings of the 100 MHz wall clock: entry, first batch multiplied, k loop
 // done, stores issued, stores acknowledged) and returns the workgroup count of that launch, or a negative value.
 extern "C" int eet_timeline_begin(int launches)
 {

@@ -186,6 +186,19 @@ def test_pair_split(gpu, tuning, cfg):
     assert small_m_shape(8, 4096, 4096, 0, True)[3] == 1 and small_m_shape(8, 4096, 4096, 2, False)[3] == 1
 
 
+@pytest.mark.parametrize("cfg", ["4,8,1,4", "5,8,1,4"])
+def test_pair_split_is_reproducible(gpu, tuning, cfg):
+    """Four workgroups share a tile's k range and whichever arrives last adds the shares: it adds them in
+    the order of the k range, not of arrival, so that repeated launches give the same bits."""
+    tuning("EET_GEMM_SMALL_M_CONFIG", cfg)
+    M, K, N = 32, 13696, 5120
+    x, u, p, s = make(M, K, N, 5)
+    xd, pd, sd = x.to(gpu), p.to(gpu), s.to(gpu)
+    first = gemm(xd, pd, sd, M, N, K).clone()
+    for rep in range(30):
+        assert torch.equal(gemm(xd, pd, sd, M, N, K), first), f"launch {rep} differs from the first"
+
+
 def test_k_split_dispatch(gpu):
     """What the table picks (no override) for a call that hands over the workspace: the k split for the O / down
     launches of both decoders at the batch sizes where it measured faster, the plain launch elsewhere."""

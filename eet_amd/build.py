@@ -27,6 +27,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
 ]

@@ -329,6 +329,12 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
     const int units = (epi == kEpiSwiglu) ? (NT / 2) * MT : NT * MT;
     half4 sc0[kMaxUnits], sc1[kMaxUnits], res[kMaxUnits];
     {
+        // The residual rows come through a buffer resource that is empty unless the epilogue adds them: the
+        // load needs no branch then (behind a branch the compiler merges the loaded registers right after it,
+        // i.e. makes the wavefront wait a whole memory latency before its first weight request).
+        [[maybe_unused]] const __amdgpu_buffer_rsrc_t res_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<_Float16 *>(residual), 0, (!CHAIN && epi == kEpiResidual) ? (unsigned)M * (unsigned)N * 2u : 0u,
+            0x00020000);
         int idx = 0;
         for (int unit = wave; unit < units; unit += WAVES, ++idx) {
             const int mt = unit % MT;
@@ -337,9 +343,11 @@ __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
             sc0[idx] = *reinterpret_cast<const half4 *>(scale + nt * 16 + 4 * g);
             if (epi == kEpiSwiglu)
                 sc1[idx] = *reinterpret_cast<const half4 *>(scale + min(nt + 1, ntiles - 1) * 16 + 4 * g);
-            if (!CHAIN && epi == kEpiResidual) {
+            if constexpr (!CHAIN) {
                 const int m = min(mt * 16 + j, M - 1);
-                res[idx] = *reinterpret_cast<const half4 *>(residual + (size_t)m * N + nt * 16 + 4 * g);
+                res[idx] = __builtin_bit_cast(
+                    half4, __builtin_amdgcn_raw_buffer_load_b64(
+                               res_rsrc, ((unsigned)m * (unsigned)N + (unsigned)(nt * 16 + 4 * g)) * 2u, 0, 0));
             }
         }
     }

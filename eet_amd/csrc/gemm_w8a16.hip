@@ -256,9 +256,12 @@ constexpr int kPairTiles = 10;   // NT * MT <= 10 tiles per group
 
 template <int NT, int RG, int WAVES, int U, bool RMS, int MODE>
 __global__ __launch_bounds__(WAVES * 64) void w8a16_small_m_kernel(
-    const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, const _Float16 *__restrict__ scale,
-    _Float16 *__restrict__ C, int M, int N, int K, const _Float16 *__restrict__ residual, int epi,
-    const _Float16 *__restrict__ rms_gamma, float rms_eps, eet::ChainLink link, PairArgs pair EET_TL_PARAM)
+    // argument order: the first 14 dwords are in SGPRs when a wavefront starts (kernel-argument preload); they
+    // hold what the first requests of the wavefront need, the rest is fetched while those are in flight
+    const _Float16 *__restrict__ A, const u32x4 *__restrict__ Wp, int M, int N, int K, int epi,
+    const _Float16 *__restrict__ residual, const _Float16 *__restrict__ rms_gamma,
+    const _Float16 *__restrict__ scale, _Float16 *__restrict__ C, float rms_eps, eet::ChainLink link,
+    PairArgs pair EET_TL_PARAM)
 {
     constexpr bool CHAIN = MODE == kChained, PAIR = MODE == kPair2 || MODE == kPair4;
     constexpr int KS = PAIR ? MODE : 1;
@@ -634,8 +637,8 @@ int launch_small_m(const GemmArgs &a)
     const int ntiles = a.N / 16;
     dim3 grid((ntiles + NT - 1) / NT), block(WAVES * 64);
     [[maybe_unused]] const int grid_of_launch = (int)grid.x;
-    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U, RMS, kPlain>), grid, block, 0, a.st, a.A, a.Wp, a.scale,
-                       a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, eet::ChainLink{}, PairArgs{} EET_TL_ARG);
+    hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U, RMS, kPlain>), grid, block, 0, a.st, a.A, a.Wp, a.M, a.N,
+                       a.K, a.epi, a.residual, a.rms_gamma, a.scale, a.C, a.rms_eps, eet::ChainLink{}, PairArgs{} EET_TL_ARG);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }
@@ -667,7 +670,7 @@ int launch_small_m_pair(const GemmArgs &a)
     pa.sums = reinterpret_cast<floatx4 *>(static_cast<char *>(a.ws) + kSplitTicketBytes);
     [[maybe_unused]] const int grid_of_launch = groups * KS;
     hipLaunchKernelGGL((w8a16_small_m_kernel<NT, RG, WAVES, U, false, KS>), dim3(groups, KS), dim3(WAVES * 64), 0, a.st,
-                       a.A, a.Wp, a.scale, a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps,
+                       a.A, a.Wp, a.M, a.N, a.K, a.epi, a.residual, a.rms_gamma, a.scale, a.C, a.rms_eps,
                        eet::ChainLink{}, pa EET_TL_ARG);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
@@ -686,11 +689,11 @@ int launch_small_m_chained(const GemmArgs &a)
         return rc;
     auto kern = w8a16_small_m_kernel<NT, RG, WAVES, U, RMS, kChained>;
     if (any_order)
-        hipExtLaunchKernelGGL(kern, grid, block, 0, a.st, nullptr, nullptr, hipExtAnyOrderLaunch, a.A, a.Wp, a.scale,
-                              a.C, a.M, a.N, a.K, a.residual, a.epi, a.rms_gamma, a.rms_eps, link, PairArgs{} EET_TL_NONE);
+        hipExtLaunchKernelGGL(kern, grid, block, 0, a.st, nullptr, nullptr, hipExtAnyOrderLaunch, a.A, a.Wp, a.M, a.N,
+                              a.K, a.epi, a.residual, a.rms_gamma, a.scale, a.C, a.rms_eps, link, PairArgs{} EET_TL_NONE);
     else
-        hipLaunchKernelGGL(kern, grid, block, 0, a.st, a.A, a.Wp, a.scale, a.C, a.M, a.N, a.K, a.residual, a.epi,
-                           a.rms_gamma, a.rms_eps, link, PairArgs{} EET_TL_NONE);
+        hipLaunchKernelGGL(kern, grid, block, 0, a.st, a.A, a.Wp, a.M, a.N, a.K, a.epi, a.residual, a.rms_gamma,
+                           a.scale, a.C, a.rms_eps, link, PairArgs{} EET_TL_NONE);
     EET_HIP_CHECK(hipGetLastError());
     return EET_OK;
 }

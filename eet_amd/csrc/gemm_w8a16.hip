@@ -819,9 +819,49 @@ bool pick_k_split(int M, int ntiles, int K, SmallMConfig *out)
     return false;
 }
 
+// Launch shapes that measured faster than both the formula's choice and the k split on the shapes of the two
+// decoders (us per launch, fused prologue / epilogue, 24 or 12 matrices in rotation, formula or split -> this):
+//   RMSnorm + QKV, 768 n-tiles (4096 -> 12288): M <= 2  11.33 -> 9.87 with NT 3, i.e. exactly one workgroup per CU
+//                                               (the formula takes NT 3 from M = 4 on)
+//   RMSnorm + QKV, 960 n-tiles (5120 -> 15360): M = 1 / 2 / 4  16.31 / 14.52 / 14.53 -> 14.75 / 13.76 / 13.89 with NT 2
+//                                               and two k-tiles per batch
+//   RMSnorm + gate|up, 1712 n-tiles (5120 -> 27392): M <= 2  24.7 -> 23.6 with NT 4; M = 16  26.1 -> 25.4 with NT 8
+//   O, 256 n-tiles, K = 4096: M = 1 / 8 / 16  4.94 / 5.21 / 6.03 -> 4.51 / 4.98 / 5.80 with 8 wavefronts and two
+//                                               k-tiles per batch instead of 16 wavefronts (M = 16: instead of the split)
+//   down, 256 n-tiles, K = 11008: M <= 4  8.81 -> 8.52 with one k-tile per batch
+//   O, 320 n-tiles, K = 5120: M = 1 / 4 / 8  7.67 / 7.64 / 7.54 -> 6.34 / 6.72 / 7.31 with NT 2 (160 workgroups of 8
+//                                               wavefronts, two k-tiles per batch) instead of the split; M = 32
+//                                               11.30 -> 10.95 with 4 wavefronts
+bool pick_measured(int M, int ntiles, int K, int epi, bool rms, SmallMConfig *out)
+{
+    if (rms && epi != kEpiSwiglu) {
+        if (ntiles == 768 && M <= 2)
+            return *out = SmallMConfig{3, 8, 1}, true;
+        if (ntiles == 960 && M <= 4)
+            return *out = SmallMConfig{2, 8, 2}, true;
+    }
+    if (rms && epi == kEpiSwiglu && ntiles == 1712 && M <= 2)
+        return *out = SmallMConfig{4, 8, 1}, true;
+    if (rms && epi == kEpiSwiglu && ntiles == 1712 && M > 8 && M <= 16)
+        return *out = SmallMConfig{8, 8, 1}, true;
+    if (!rms && epi != kEpiSwiglu) {
+        if (ntiles == 256 && K <= 8192 && M <= 16)
+            return *out = SmallMConfig{1, 8, 2}, true;
+        if (ntiles == 256 && K > 8192 && M <= 4)
+            return *out = SmallMConfig{1, 16, 1}, true;
+        if (ntiles == 320 && K <= 8192 && M <= 8)
+            return *out = SmallMConfig{2, 8, 2}, true;
+        if (ntiles == 320 && K <= 8192 && M > 16)
+            return *out = SmallMConfig{2, 4, 2}, true;
+    }
+    return false;
+}
+
 SmallMConfig pick_small_m(int M, int N, int K, int epi, bool rms, bool may_split)
 {
     const int ntiles = N / 16;
+    if (SmallMConfig measured; pick_measured(M, ntiles, K, epi, rms, &measured))
+        return measured;
     if (SmallMConfig split; may_split && !rms && epi != kEpiSwiglu && pick_k_split(M, ntiles, K, &split))
         return split;
     int best_nt = 0;

@@ -201,15 +201,26 @@ def test_pair_split_is_reproducible(gpu, tuning, cfg):
 
 def test_k_split_dispatch(gpu):
     """What the table picks (no override) for a call that hands over the workspace: the k split for the O / down
-    launches of both decoders at the batch sizes where it measured faster, the plain launch elsewhere."""
-    assert small_m_shape(16, 4096, 4096, 1, False) == (2, 4, 2, 2)       # LLaMA O, M = 16
-    assert small_m_shape(32, 4096, 11008, 1, False) == (4, 8, 1, 4)      # LLaMA down, M = 32
-    assert small_m_shape(8, 4096, 4096, 1, False)[3] == 1                # M <= 8: not on the LLaMA shapes
-    assert small_m_shape(8, 5120, 5120, 1, False) == (5, 8, 1, 4)        # Baichuan O: 320 n-tiles as 64 groups x 4
-    assert small_m_shape(32, 5120, 5120, 1, False)[3] == 1               # ... but not at M = 32 with the short k range
+    launches of both decoders at the batch sizes where it measured faster, the plain launch elsewhere; and the
+    launch shapes measured for the decoders' other launches at one and two rows."""
+    assert small_m_shape(32, 4096, 4096, 1, False) == (2, 8, 1, 2)       # LLaMA O, M = 32
+    assert small_m_shape(16, 4096, 4096, 1, False) == (1, 8, 2, 1)       # ... up to M = 16 a plain launch measured faster
+    assert small_m_shape(16, 4096, 11008, 1, False) == (4, 4, 1, 4)      # LLaMA down, M = 16 / 32
+    assert small_m_shape(32, 4096, 11008, 1, False) == (4, 8, 1, 4)
+    assert small_m_shape(8, 4096, 11008, 1, False)[3] == 1               # M <= 8: not on the LLaMA shapes
+    assert small_m_shape(16, 5120, 5120, 1, False) == (5, 8, 1, 4)       # Baichuan O: 320 n-tiles as 64 groups x 4
+    assert small_m_shape(8, 5120, 5120, 1, False) == (2, 8, 2, 1)        # ... up to M = 8 a plain launch measured faster
+    assert small_m_shape(32, 5120, 5120, 1, False) == (2, 4, 2, 1)       # ... and not at M = 32 with the short k range
     assert small_m_shape(32, 5120, 13696, 1, False) == (5, 8, 1, 4)
+    assert small_m_shape(8, 5120, 13696, 1, False) == (5, 8, 1, 4)
     assert small_m_shape(16, 12288, 4096, 0, True)[3] == 1               # never with the RMSnorm prologue
     assert small_m_shape(16, 4112, 4096, 1, False)[3] == 1               # other channel counts keep the table's choice
+    assert small_m_shape(1, 12288, 4096, 0, True) == (3, 8, 1, 1)        # RMSnorm + QKV: one workgroup per CU from M = 1 on
+    assert small_m_shape(8, 12288, 4096, 0, True) == (3, 8, 1, 1)
+    assert small_m_shape(1, 15360, 5120, 0, True) == (2, 8, 2, 1)
+    assert small_m_shape(16, 27392, 5120, 2, True) == (8, 8, 1, 1)
+    assert small_m_shape(2, 27392, 5120, 2, True) == (4, 8, 1, 1)
+    assert small_m_shape(4, 4096, 11008, 1, False) == (1, 16, 1, 1)
 
 
 LARGE_M_TILES = ["8,4", "4,5", "4,4", "4,2", "2,2"]   # m-tiles, n-tiles per wavefront

@@ -190,7 +190,7 @@ def test_recorded_step_survives_workspace_regrowth_and_resyncs(gpu):
 
 
 def test_graph_replays_with_the_k_split_match_eager(gpu):
-    """At batch 16 the O and down projections of a LLaMA-7B-width layer run with the k split (two and four
+    """At batch 16 the down projection of a LLaMA-7B-width layer runs with the k split (four
     workgroups share a tile group and exchange partial sums through a named workspace whose counters must be
     zero): the recorded step replays that workspace's pointer, so replays must leave the counters as eager
     calls do.  Token for token against the eager loop, and an eager run AFTER the replays on the same
@@ -198,8 +198,8 @@ def test_graph_replays_with_the_k_split_match_eager(gpu):
     import ctypes
     from eet_amd._lib import check, lib
     v = [ctypes.c_int(0) for _ in range(4)]
-    check(lib().eet_gemm_w8a16_small_m_shape(16, 4096, 4096, 1, 0, *[ctypes.byref(x) for x in v]))
-    assert v[3].value > 1 and lib().eet_gemm_w8a16_workspace(16, 4096, 4096, 1) > 0, "the k split is expected here"
+    check(lib().eet_gemm_w8a16_small_m_shape(16, 4096, 11008, 1, 0, *[ctypes.byref(x) for x in v]))
+    assert v[3].value > 1 and lib().eet_gemm_w8a16_workspace(16, 4096, 11008, 1) > 0, "the k split is expected here"
     cfg = D.DecoderConfig(num_layers=1, hidden=4096, heads=32, d_ff=11008, vocab=512, eps=1e-6, alibi=False, max_batch=16,
                           max_prompt=8, max_full_seq=24)
     sd, _ = D.random_state_dict(cfg, seed=11)

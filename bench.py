@@ -676,8 +676,8 @@ def recorded_traffic(M, layers):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--m", type=int, default=8, help="activation rows of the headline GEMM pass")
     ap.add_argument("--layers", type=int, default=LLAMA["layers"])
     ap.add_argument("--gen", type=int, default=128, help="tokens to greedy-decode in the decoder leg (0 = skip)")

@@ -756,7 +756,7 @@ int dispatch_small_m(SmallMConfig cfg, const GemmArgs &a, bool dry)
     }
         EET_CASE_CHAIN(1, 8, 2) EET_CASE_CHAIN(1, 16, 2) EET_CASE_CHAIN(1, 16, 1)
         EET_CASE_CHAIN(2, 8, 2) EET_CASE_CHAIN(2, 8, 1) EET_CASE_CHAIN(3, 8, 1)
-        EET_CASE_CHAIN(4, 8, 1) EET_CASE_CHAIN(6, 8, 1) EET_CASE_CHAIN(8, 8, 1)
+        EET_CASE_CHAIN(4, 8, 1) EET_CASE_CHAIN(6, 8, 1) EET_CASE_CHAIN(8, 8, 1) EET_CASE_CHAIN(2, 4, 2)
 #undef EET_CASE_CHAIN
         return kNoVariant;
     }

@@ -1012,6 +1012,18 @@ extern "C" int eet_gemm_w8a16_small_m_shape(int M, int N, int K, int epilogue, i
     a.ws_bytes = ~size_t(0);
     const SmallMConfig cfg = resolve_small_m(a);
     *nt = cfg.nt, *waves = cfg.waves, *k_tiles_per_batch = cfg.u, *k_split = cfg.ksplit;
+    // The library must hold a kernel for what the table answers in every form of the call: with the
+    // workspace (above), without it, and chained.  Decided without launching.
+    GemmArgs bare = a, chained = a;
+    bare.ws = nullptr, bare.ws_bytes = 0;
+    chained.ws = nullptr, chained.ws_bytes = 0, chained.chain = eet::kChainNext;
+    for (const GemmArgs *form : {&a, &bare, &chained}) {
+        const SmallMConfig c = resolve_small_m(*form);
+        EET_REQUIRE(dispatch_by_rows(c, *form, true) == EET_OK, EET_ERR_INVALID_ARGUMENT,
+                    "eet_gemm_w8a16_small_m_shape: no small-M kernel for nt=%d waves=%d u=%d ksplit=%d (M=%d N=%d K=%d epilogue %d%s%s)",
+                    c.nt, c.waves, c.u, c.ksplit, M, N, K, epilogue, rms_prologue ? ", RMSnorm prologue" : "",
+                    form == &chained ? ", chained" : form == &bare ? ", no workspace" : "");
+    }
     return EET_OK;
 }
 

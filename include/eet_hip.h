@@ -171,7 +171,10 @@ int eet_gemm_w8a16_fused(const void *A, const void *Wpacked, const void *scale, 
  * over the workspace eet_gemm_w8a16_workspace asks for -- without it, 1) -- the tuning
  * override EET_GEMM_SMALL_M_CONFIG when a kernel of that shape exists for the
  * call, otherwise the table's choice.  For sweeps and for tests that must know
- * which variant ran.  The reference's counterpart is the CutlassGemmConfig its
+ * which variant ran.  It also checks, on the host, that the library holds a kernel
+ * for what the table answers in every form of the call (with the workspace,
+ * without it, chained) and fails with EET_ERR_INVALID_ARGUMENT if not.  The
+ * reference's counterpart is the CutlassGemmConfig its
  * heuristic returns (cutlass_heuristic.cc:106-207). */
 int eet_gemm_w8a16_small_m_shape(int M, int N, int K, int epilogue, int rms_prologue, int *nt,
                                  int *waves, int *k_tiles_per_batch, int *k_split);

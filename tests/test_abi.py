@@ -162,3 +162,22 @@ def test_tuning_keys():
     assert b"nt,waves,u" in L.eet_last_error()
     assert L.eet_set_tuning(b"EET_NO_SUCH_KEY", b"1") != 0
     assert b"unknown key" in L.eet_last_error()
+
+
+def test_every_table_answer_has_a_kernel():
+    """The small-M launch-shape table (formula, measured shapes, k split) only answers with shapes the library
+    holds a kernel for -- plain, without the workspace and chained: the query decides this on the host, for
+    every row count and a wide range of channel counts, with every prologue / epilogue."""
+    L = _lib.lib()
+    q = [ctypes.c_int() for _ in range(4)]
+    widths = sorted(set(list(range(16, 2049, 16)) + [n * 16 for n in (160, 192, 200, 230, 240, 255, 256, 257, 300, 320, 344, 384,
+                                                                         428, 480, 512, 640, 688, 768, 856, 960, 1024, 1376,
+                                                                         1712, 2000, 2048, 2752, 4096)]))
+    for K in (64, 4096, 5120, 11008, 13696):
+        for N in widths:
+            for M in (1, 2, 3, 4, 7, 8, 9, 16, 17, 24, 32):
+                for epi, rms in ((0, 0), (1, 0), (0, 1), (1, 1), (2, 1), (2, 0)):
+                    if epi == 2 and N % 32:
+                        continue
+                    rc = L.eet_gemm_w8a16_small_m_shape(M, N, K, epi, rms, *[ctypes.byref(x) for x in q])
+                    assert rc == 0, L.eet_last_error().decode()

@@ -107,7 +107,8 @@ def alibi_table(H, S, gpu):
     return (slopes[:, None] * torch.arange(S, dtype=torch.float32)[None, :]).half().to(gpu)
 
 
-@pytest.mark.parametrize("B,H,S,alibi", [(8, 32, 1024, False), (8, 40, 2048, True), (8, 40, 2048, False)])
+@pytest.mark.parametrize("B,H,S,alibi", [(8, 32, 1024, False), (8, 40, 2048, True), (8, 40, 2048, False),
+                                         (1, 32, 8192, False), (1, 8, 6001, True)])   # the last two: past the reference's 4096 / 2048 caps
 def test_prefill_attention_full_grid_uniform_keys(gpu, B, H, S, alibi):
     """Every (b, h, i) of the launch the configuration makes.  All keys of a (b, h) pair are the same row, so
     the scores of a query are equal and its weights are softmax(bias[:i+1]) (uniform without a bias)."""

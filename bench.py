@@ -96,6 +96,12 @@ def bench_lib():
     h.eet_timeline_launches.restype = i
     h.eet_timeline_read.restype = i
     h.eet_timeline_read.argtypes = [i, vp]
+    h.eet_timeline_mmha_decode.restype = i           # eet_mmha_decode with clock readings in the kernel
+    h.eet_timeline_mmha_decode.argtypes = [vp, vp, vp, ctypes.c_long, vp, vp, vp, vp, vp, i, i, i, i, i, vp, vp, sz, vp]
+    h.eet_timeline_attn_begin.restype = i
+    h.eet_timeline_attn_begin.argtypes = [i]
+    h.eet_timeline_attn_read.restype = i
+    h.eet_timeline_attn_read.argtypes = [i, vp]
     return h
 
 
@@ -657,6 +663,74 @@ def attention_bench(torch, lib, dev, iters=20):
     return out
 
 
+def attention_timeline(torch, dev, launches=12):
+    """Where the time of a decode-attention launch goes, read inside the kernel (bench-only build of the same
+    source): back-to-back launches over caches in rotation at the two decoder shapes; the second of two recorded
+    passes is analysed."""
+    import ctypes
+    import numpy as np
+    B_ = bench_lib()
+    st = torch.cuda.current_stream()
+    out = {}
+    for name, B, H, step, alibi in (("llama7b B=8 step=1088", 8, 32, 1088, False),
+                                    ("baichuan13b B=32 step=2176 alibi", 32, 40, 2176, True)):
+        dh, cap = 128, step + 1
+        g = torch.Generator(device=dev).manual_seed(step)
+        per = 2 * B * H * cap * dh * 2
+        ncache = max(2, int(600e6 // per) + 1)
+        caches = [(torch.randn(B, H, cap, dh, generator=g, device=dev).half(),
+                   torch.randn(B, H, cap, dh, generator=g, device=dev).half()) for _ in range(ncache)]
+        q, k, v = [torch.randn(B, H, dh, generator=g, device=dev).half() for _ in range(3)]
+        ctx = torch.empty(B, H * dh, dtype=torch.float16, device=dev)
+        bias = (torch.rand(H, step, generator=g, device=dev) * 8).half() if alibi else None
+        if B_.eet_timeline_attn_begin(2 * launches):
+            return {"error": "eet_timeline_attn_begin failed"}
+        torch.cuda.synchronize()
+        for i in range(2 * launches):
+            kc, vc = caches[i % ncache]
+            rc = B_.eet_timeline_mmha_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), 0, kc.data_ptr(), vc.data_ptr(),
+                                             ctx.data_ptr(), bias.data_ptr() if alibi else None, None, B, H, dh, step,
+                                             cap, None, None, 0, st.cuda_stream)
+            if rc:
+                return {"error": f"eet_timeline_mmha_decode returned {rc}"}
+        torch.cuda.synchronize()
+        buf = np.zeros(2048 * 8, dtype=np.uint64)
+        stamps = []
+        for l in range(launches - 1, 2 * launches):
+            wgs = B_.eet_timeline_attn_read(l, buf.ctypes.data_as(ctypes.c_void_p))
+            if wgs <= 0:
+                return {"error": f"eet_timeline_attn_read({l}) returned {wgs}"}
+            stamps.append(buf[: wgs * 8].reshape(wgs, 8).astype(np.int64).copy())
+        rows = []
+        for i in range(1, len(stamps) - 1):
+            prev, cur, nxt = stamps[i - 1], stamps[i], stamps[i + 1]
+            t0 = cur[:, 0].min()
+            rows.append([nxt[:, 0].min() - t0,                    # period
+                         t0 - prev[:, 6].max(),                   # idle: last acknowledged store of the predecessor -> first entry
+                         cur[:, 0].max() - t0,                    # entry spread
+                         (cur[:, 1] - cur[:, 0]).mean(),          # entry -> new token handled, ring requested
+                         (cur[:, 2] - cur[:, 0]).mean(),          # entry -> first row consumed
+                         (cur[:, 3] - t0).min(), (cur[:, 3] - t0).mean(), (cur[:, 3] - t0).max(),   # first wavefront through its rows
+                         (cur[:, 4] - cur[:, 3]).mean(),          # ... -> all wavefronts of the workgroup through
+                         (cur[:, 4] - t0).max(),                  # the last workgroup's barrier
+                         (cur[:, 5] - cur[:, 4]).mean(),          # merge of the streams, result stores issued
+                         (cur[:, 6] - cur[:, 5]).mean(),          # stores acknowledged
+                         cur[:, 6].max() - t0])
+        a = np.mean(np.array(rows, dtype=np.float64), axis=0) / 100.0
+        out[name] = {"launches": len(rows), "workgroups": int(stamps[1].shape[0]), "period_us": round(a[0], 2),
+                     "idle_before_first_entry_us": round(a[1], 2), "entry_spread_us": round(a[2], 2),
+                     "entry_to_ring_requested_us": round(a[3], 2), "entry_to_first_row_consumed_us": round(a[4], 2),
+                     "first_wavefront_through_after_first_entry_us": {"first": round(a[5], 2), "mean": round(a[6], 2), "last": round(a[7], 2)},
+                     "wait_for_the_other_wavefronts_us": round(a[8], 2), "last_workgroup_barrier_after_first_entry_us": round(a[9], 2),
+                     "merge_of_the_streams_us": round(a[10], 2), "store_acknowledge_us": round(a[11], 2),
+                     "first_entry_to_last_acknowledge_us": round(a[12], 2)}
+        del caches
+    out["what"] = ("clock readings inside the decode-attention kernel (bench-only build with -DEET_TIMELINE of the same "
+                   "source; thread 0 of each workgroup, 100 MHz wall clock), back-to-back launches over caches in rotation, "
+                   "second of two recorded passes")
+    return out
+
+
 def recorded_traffic(M, layers):
     """HBM-side bytes per launch of the headline pass as recorded in profiles/ (a line
     'traffic_bytes_per_launch M=<M> layers=<n>: <bytes>' in the pmc summary), or None."""
@@ -840,6 +914,11 @@ def main():
         result["prefill_attention"] = prefill_attention_bench(torch, L, dev)
     if (not args.no_sweep and not only) or "decode_attention" in only:
         result["decode_attention"] = attention_bench(torch, L, dev)
+        if not args.no_timeline:
+            try:
+                result["decode_attention_timeline"] = attention_timeline(torch, dev)
+            except (RuntimeError, OSError, AttributeError) as e:   # measurement only: never ends the run
+                result["decode_attention_timeline"] = {"error": str(e)}
     if (not args.no_sweep and not only) or "packer_device" in only:
         result["packer_device"] = device_packer_bench(torch, eet, L, dev)
 

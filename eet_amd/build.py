@@ -1,7 +1,7 @@
 """Builds libeet_hip.so (HIP kernels + C ABI + host packer) and libeet_bench.so (measurement only, no
 part of the operator interface: the read-only streaming probe that bench.py times beside the GEMM
-pass, and the dequant-GEMM source compiled a second time with -DEET_TIMELINE, i.e. with clock
-readings inside the small-M kernel, under eet_timeline_* names) for gfx950 with hipcc.
+pass, and the dequant-GEMM and decode-attention sources compiled a second time with -DEET_TIMELINE, i.e.
+with clock readings inside the kernels, under eet_timeline_* names) for gfx950 with hipcc.
 
 Run as `python -m eet_amd.build`.  The libraries are built in-tree, next to this
 file, so that they travel with the source tree.
@@ -20,8 +20,8 @@ BENCH_LIB = os.path.join(HERE, "libeet_bench.so")
 SOURCES = ["packer.cc", "tuning.cc", "decode_ops.cc", "chain.hip", "packer_device.hip", "gemm_w8a16.hip",
            "gemm_w8a16_large.hip", "mmha_decode.hip", "prefill_attention.hip", "glue.hip"]
 BENCH_SOURCES = ["probe.hip"]
-TIMELINE_SOURCE = "gemm_w8a16.hip"        # compiled again with -DEET_TIMELINE for libeet_bench.so
-TIMELINE_OBJ = "gemm_w8a16.timeline.o"
+# compiled again with -DEET_TIMELINE for libeet_bench.so
+TIMELINE_SOURCES = {"gemm_w8a16.hip": "gemm_w8a16.timeline.o", "mmha_decode.hip": "mmha_decode.timeline.o"}
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -48,11 +48,12 @@ def build(verbose=True):
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
         objs.append(obj)
-    cmd = [HIPCC] + [f for f in FLAGS if f != "-shared"] + ["-DEET_TIMELINE", "-x", "hip", "-c", os.path.join(CSRC, TIMELINE_SOURCE),
-                                                           "-o", os.path.join(HERE, "_obj", TIMELINE_OBJ)]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    procs.append((TIMELINE_SOURCE + " (timeline)", subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    for src, obj in TIMELINE_SOURCES.items():
+        cmd = [HIPCC] + [f for f in FLAGS if f != "-shared"] + ["-DEET_TIMELINE", "-x", "hip", "-c", os.path.join(CSRC, src),
+                                                               "-o", os.path.join(HERE, "_obj", obj)]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src + " (timeline)", subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
     failed = False
     for src, p in procs:
         out, _ = p.communicate()
@@ -68,7 +69,8 @@ def build(verbose=True):
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + \
               [os.path.join(HERE, "_obj", src + ".o") for src in srcs]
         if lib == BENCH_LIB:   # the instrumented GEMM uses the operator library's dispatch tables and error slot
-            cmd += [os.path.join(HERE, "_obj", TIMELINE_OBJ), "-L" + HERE, "-leet_hip", "-Wl,-rpath,$ORIGIN"]
+            cmd += [os.path.join(HERE, "_obj", obj) for obj in TIMELINE_SOURCES.values()]
+            cmd += ["-L" + HERE, "-leet_hip", "-Wl,-rpath,$ORIGIN"]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)

@@ -17,12 +17,51 @@
 // workgroups (the reference runs one block per head); each then writes an
 // un-normalised partial (max, sum, acc[dh]) and a second small kernel merges
 // them.  There is no per-launch limit on step.
+#if defined(EET_TIMELINE)
+// Bench-only build of this file (linked into libeet_bench.so): the same kernels with clock readings per
+// workgroup, under entry-point names of their own.
+#define eet_rope_table eet_timeline_rope_table
+#define eet_mmha_decode_workspace eet_timeline_mmha_decode_workspace
+#define eet_mmha_decode eet_timeline_mmha_decode
+#define eet_step_advance eet_timeline_step_advance
+#define eet_mmha_decode_replayable_workspace eet_timeline_mmha_decode_replayable_workspace
+#define eet_mmha_decode_replayable eet_timeline_mmha_decode_replayable
+#define eet_mmha_decode_static_capacity eet_timeline_mmha_decode_static_capacity
+#define eet_mmha_decode_static eet_timeline_mmha_decode_static
+#endif
 #include <hip/hip_runtime.h>
 
 #include <cmath>
 
 #include "common.h"
 #include "tuning.h"
+
+#if defined(EET_TIMELINE)
+#define EET_ATL_PARAM , unsigned long long *tl
+#define EET_ATL_ARG , attn_timeline_next((int)(grid.x * grid.y))
+#define EET_ATL_STAMP(i)                                   \
+    do {                                                   \
+        if (tl != nullptr && threadIdx.x == 0)             \
+            tl_t[i] = wall_clock64();                      \
+    } while (0)
+namespace {
+constexpr int kAtlStamps = 8, kAtlMaxWgs = 2048;
+unsigned long long *g_atl_buf = nullptr;   // [launch][kAtlMaxWgs][kAtlStamps], device memory
+int g_atl_cap = 0, g_atl_n = 0;
+int g_atl_grid[1024];
+unsigned long long *attn_timeline_next(int workgroups)
+{
+    if (g_atl_buf == nullptr || g_atl_n >= g_atl_cap || g_atl_n >= 1024 || workgroups > kAtlMaxWgs)
+        return nullptr;
+    g_atl_grid[g_atl_n] = workgroups;
+    return g_atl_buf + (size_t)(g_atl_n++) * kAtlMaxWgs * kAtlStamps;
+}
+}  // namespace
+#else
+#define EET_ATL_PARAM
+#define EET_ATL_ARG
+#define EET_ATL_STAMP(i)
+#endif
 
 namespace {
 
@@ -85,8 +124,12 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
     long qkv_stride, _Float16 *__restrict__ k_cache, _Float16 *__restrict__ v_cache, _Float16 *__restrict__ ctx,
     const _Float16 *__restrict__ alibi, const int64_t *__restrict__ pad, float *__restrict__ partial, int H,
     int step, int T_cap, int nsplit, float scale, const float *__restrict__ rope_row,
-    const int *__restrict__ step_dev, int alibi_ld_arg)
+    const int *__restrict__ step_dev, int alibi_ld_arg EET_ATL_PARAM)
 {
+#if defined(EET_TIMELINE)
+    unsigned long long tl_t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#endif
+    EET_ATL_STAMP(0);
     // Replayable form (a launch recorded into a HIP graph): the step lives in device
     // memory, rope_row is the base of the whole rotary table and the bias rows have a
     // fixed leading dimension, so that the same recorded arguments serve every step.
@@ -102,7 +145,7 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
     constexpr int NS = slices_per_row(DH);   // of which this many hold a slice
     constexpr int RPB = THREADS / LPR;       // row streams of the block (one per group of LPR lanes)
     __shared__ float accs[RPB][DH + 1];
-    __shared__ float stream_m[RPB], stream_l[RPB];
+    __shared__ float stream_m[RPB], stream_l[RPB], stream_w[RPB], merged_max;
 
     const int split = blockIdx.y;
     const int bh = blockIdx.x;
@@ -237,6 +280,7 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
         }
     }
     __builtin_amdgcn_sched_barrier(0);
+    EET_ATL_STAMP(1);   // new token rotated and appended, the ring requested
     float m_run = -INFINITY, l_run = 0.f;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const int iters = (n + RPB - 1) / RPB;  // the same for every stream of the workgroup
@@ -265,8 +309,13 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
             __builtin_amdgcn_sched_barrier(0);
             request(u, i0 + u + UN);
             __builtin_amdgcn_sched_barrier(0);
+#if defined(EET_TIMELINE)
+            if (i0 == 0 && u == 0)
+                EET_ATL_STAMP(2);   // the first row of this stream consumed
+#endif
         }
     }
+    EET_ATL_STAMP(3);   // the first wavefront's streams are through their rows
 #else
     float m_run = -INFINITY, l_run = 0.f;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -283,16 +332,27 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
         stream_l[rs] = l_run;
     }
     __syncthreads();
-    if (tid < DH) {
+    EET_ATL_STAMP(4);   // every wavefront of the workgroup is through
+    // The weight of every stream in the merge, exp(m - max over the streams), is computed once, by one lane per
+    // stream, and the lanes that own an output element then only multiply and add (with the exponentials inside
+    // their loop the merge took 1.3 us of a 24 us launch).
+    if (tid < RPB) {
         float lmax = -INFINITY;
-#pragma unroll 4
+#pragma unroll 8
         for (int r = 0; r < RPB; ++r)
             lmax = fmaxf(lmax, stream_m[r]);
+        const float mr = stream_m[tid];
+        stream_w[tid] = (mr == -INFINITY) ? 0.f : __expf(mr - lmax);
+        if (tid == 0)
+            merged_max = lmax;
+    }
+    __syncthreads();
+    if (tid < DH) {
+        const float lmax = merged_max;
         float s = 0.f, lsum = 0.f;
-#pragma unroll 4
+#pragma unroll 8
         for (int r = 0; r < RPB; ++r) {
-            const float mr = stream_m[r];
-            const float w = (mr == -INFINITY) ? 0.f : __expf(mr - lmax);
+            const float w = stream_w[r];
             lsum += w * stream_l[r];
             s += w * accs[r][tid];
         }
@@ -308,6 +368,16 @@ __global__ __launch_bounds__(THREADS) void mmha_decode_split_kernel(
             }
         }
     }
+#if defined(EET_TIMELINE)
+    EET_ATL_STAMP(5);   // streams merged, result stores issued
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    EET_ATL_STAMP(6);   // ... and acknowledged
+    if (tl != nullptr && threadIdx.x == 0) {
+        unsigned long long *o = tl + (size_t)(blockIdx.y * gridDim.x + blockIdx.x) * kAtlStamps;
+        for (int i = 0; i < 8; ++i)
+            o[i] = tl_t[i];
+    }
+#endif
 }
 
 template <int DH>
@@ -380,7 +450,7 @@ int launch_split(const void *q, const void *k, const void *v, long qkv_stride, v
                        static_cast<const _Float16 *>(v), qkv_stride, static_cast<_Float16 *>(kc),
                        static_cast<_Float16 *>(vc), static_cast<_Float16 *>(ctx),
                        static_cast<const _Float16 *>(alibi), pad, static_cast<float *>(ws), H, step, T_cap, nsplit,
-                       scale, rope_row, step_dev, alibi_ld);
+                       scale, rope_row, step_dev, alibi_ld EET_ATL_ARG);
     EET_HIP_CHECK(hipGetLastError());
     if (nsplit > 1) {
         hipLaunchKernelGGL((mmha_decode_merge_kernel<DH>), dim3(B * H), dim3(DH), 0, st,
@@ -604,3 +674,38 @@ extern "C" int eet_mmha_decode_static(const void *q, const void *k, const void *
     return run_mmha(q, k, v, qkv_stride, k_cache, v_cache, ctx, alibi, pad, B, H, dh, step, T_cap, rope_cos_sin,
                     partials, plan, static_cast<hipStream_t>(stream));
 }
+
+#if defined(EET_TIMELINE)
+// Bench-only: recording starts with a device buffer for `launches` launches; every decode-attention launch made
+// through the eet_timeline_mmha_* entry points from then on fills the next slot.  eet_timeline_attn_read
+// synchronises the device, copies slot `launch` ([workgroup][8] readings of the 100 MHz wall clock: entry, ring
+// requested, first row consumed, first wavefront through its rows, all wavefronts through, result stores issued,
+// stores acknowledged) and returns the workgroup count of that launch, or a negative value.
+extern "C" int eet_timeline_attn_begin(int launches)
+{
+    if (g_atl_buf != nullptr && g_atl_cap < launches) {
+        (void)hipFree(g_atl_buf);
+        g_atl_buf = nullptr;
+    }
+    if (g_atl_buf == nullptr) {
+        EET_HIP_CHECK(hipMalloc(&g_atl_buf, (size_t)launches * kAtlMaxWgs * kAtlStamps * sizeof(unsigned long long)));
+        g_atl_cap = launches;
+    }
+    EET_HIP_CHECK(hipMemset(g_atl_buf, 0, (size_t)g_atl_cap * kAtlMaxWgs * kAtlStamps * sizeof(unsigned long long)));
+    g_atl_n = 0;
+    return EET_OK;
+}
+
+extern "C" int eet_timeline_attn_read(int launch, unsigned long long *host_dst)
+{
+    if (launch < 0 || launch >= g_atl_n || host_dst == nullptr)
+        return -1;
+    if (hipDeviceSynchronize() != hipSuccess)
+        return -2;
+    const int wgs = g_atl_grid[launch];
+    if (hipMemcpy(host_dst, g_atl_buf + (size_t)launch * kAtlMaxWgs * kAtlStamps,
+                  (size_t)wgs * kAtlStamps * sizeof(unsigned long long), hipMemcpyDeviceToHost) != hipSuccess)
+        return -2;
+    return wgs;
+}
+#endif
